@@ -847,7 +847,8 @@ class ModelRunner:
 class HybridModelRunner(ModelRunner):
     """Runner of layer-list decoders (``models/hybrid.py``): the same plans, graphs, sampler and bookkeeping as
     ``ModelRunner``; per layer a paged window cache (attention mixers; key and value sizes from the layer) or a set
-    of fp32 state slots (recurrent mixers), an fp32 residual stream normalised after every sum.
+    of fp32 state slots (recurrent mixers), an fp32 residual stream (normalised after every sum, between two norms, or
+    read through one norm by both sublayers of a layer, as the design says).
 
     Prompt portions and decoded tokens run the same kernels: attention reads keys and values from the pages only
     (the portion's own tokens are written first), so a position's result does not depend on how its prompt was cut;
@@ -868,7 +869,8 @@ class HybridModelRunner(ModelRunner):
         assert kv_dtype is None, "layer-list decoders keep their caches in the model's dtype"
         self.hq = self.hkv = 1
         self.sandwich = bool(getattr(self.model, "sandwich", False))
-        self.keeps_positions = self.sandwich
+        self.parallel = bool(getattr(self.model, "parallel", False))
+        self.keeps_positions = self.sandwich or self.parallel
         # one cache / state per layer RUN: a layer that runs several times keeps every pass apart
         self.layer_runs = list(getattr(self.model, "layer_runs", range(len(self.model.layers))))
         self.kv, self.state = [], []
@@ -877,8 +879,16 @@ class HybridModelRunner(ModelRunner):
             blk = self.model.layers[li]
             if blk.kind == "attention":
                 G, D, V = blk.mix.cache_shape()
+                if hasattr(blk.mix, "prepare"):  # mixers that rotate by position
+                    blk.mix.prepare(self.max_context + 1, tables, self.device)
                 self.kv.append(wattn.alloc_window_cache(self.num_pages, G, D, V, self.dtype, self.device))
                 self.state.append(None)
+            elif blk.kind == "lightning":
+                from ..ops import lightning as lightning_ops
+
+                H, D, V = blk.mix.state_shape()
+                self.kv.append(None)
+                self.state.append(lightning_ops.alloc_state(self.n_state_slots, H, D, V, self.device))
             elif blk.kind == "latent_attention":
                 R, P = blk.mix.cache_shape()
                 blk.mix.prepare(self.max_context + 1, tables)
@@ -896,7 +906,7 @@ class HybridModelRunner(ModelRunner):
         self._neg1 = torch.full((1,), -1, dtype=torch.int32, device=self.device)
 
     def _embed(self, ids: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
-        if self.sandwich:  # the embedding needs the rows of the plan: `_run_layers` computes it
+        if self.sandwich or self.parallel:  # the fp32 stream starts in `_run_layers`, from the token ids
             return ids
         return self.model.embed_tokens(ids, pos)
 
@@ -918,6 +928,8 @@ class HybridModelRunner(ModelRunner):
         cfg = self.cfg
         if self.sandwich:
             return self._run_layers_sandwich(xc, st)
+        if self.parallel:
+            return self._run_layers_parallel(xc, st)
         x32 = xc.float() if xc.dtype != torch.float32 else xc.clone()
         alpha, eps = float(cfg.postln_alpha), float(cfg.rms_norm_eps)
         trace = getattr(self, "layer_trace", None)
@@ -955,9 +967,39 @@ class HybridModelRunner(ModelRunner):
                 trace.append(x32.clone())
         return x32
 
+    def _run_layers_parallel(self, ids: torch.Tensor, st) -> torch.Tensor:
+        """Token ids -> fp32 residual stream after the last layer. One kernel closes a layer (stream += mixer output +
+        feed-forward output) and opens the next (its norm, in the compute dtype and - for layers whose router reads
+        it - in fp32)."""
+        from ..ops import parallel_block as pb
+
+        model, eps = self.model, float(self.cfg.rms_norm_eps)
+        x32 = pb.embed_scaled(ids, model.embed, float(self.cfg.embed_scale))
+        blocks = [model.layers[li] for li in self.layer_runs]
+        trace = getattr(self, "layer_trace", None)
+        st.v_first = None
+        _, h32, hc = pb.sum_norm(x32, None, None, blocks[0].norm1, eps, self.dtype, want32=blocks[0].needs32)
+        for ri, blk in enumerate(blocks):
+            y_mix, y_ff = blk.step(hc, h32, st, self.kv[ri], self.state[ri])
+            nxt = blocks[ri + 1] if ri + 1 < len(blocks) else None
+            x32, h32, hc = pb.sum_norm(x32, y_mix, y_ff, nxt.norm1 if nxt is not None else None, eps, self.dtype,
+                                       want32=nxt is not None and nxt.needs32)
+            if trace is not None:
+                trace.append(x32.clone())
+        return x32
+
     def _final_logits(self, h, residual, fp32: bool = False) -> torch.Tensor:
         from ..ops.post_norm import scaled_add_norm
 
+        if self.parallel:
+            from ..ops import parallel_block as pb
+
+            want32 = fp32 or self.keep_logits
+            _, x32, xc = pb.sum_norm(h.contiguous(), None, None, self.model.norm, float(self.cfg.rms_norm_eps),
+                                     self.dtype, want32=want32)
+            if want32:
+                return F.linear(x32, self.model.head_weight.float())
+            return F.linear(xc, self.model.head_weight)
         if self.sandwich:
             from ..ops import sandwich as sw
 
@@ -1003,7 +1045,7 @@ class HybridModelRunner(ModelRunner):
             return nsplit, ws
         mixers = [blk.mix for blk in self.model.layers if blk.kind == "attention"]
         if mixers and self.device.type == "cuda":
-            nsplit = max(wattn.decode_splits(Bp, m.shape.window, self.max_context) for m in mixers)
+            nsplit = max(wattn.decode_splits(Bp, m.shape.window, self.max_context, m.shape.keep_first) for m in mixers)
             if nsplit > 1:
                 hv = max(m.H * m.V for m in mixers)
                 hh = max(m.H for m in mixers)

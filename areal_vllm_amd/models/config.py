@@ -13,7 +13,7 @@ from typing import Any, Dict, List, Optional
 
 
 # config.json "architecture" -> reader in models/hybrid.py (designs given as a list of layers)
-LAYER_LIST_DESIGNS = {"Kuzanex": "kuzanex_config", "Lufivik": "lufivik_config"}
+LAYER_LIST_DESIGNS = {"Kuzanex": "kuzanex_config", "Lufivik": "lufivik_config", "Pobelorn": "pobelorn_config"}
 
 
 @dataclasses.dataclass

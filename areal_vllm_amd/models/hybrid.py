@@ -13,10 +13,21 @@ Mixer:      attention through a shared low-rank latent (the cache holds the late
 ff:         routed experts, gated units with clamped pre-activations, softmax router weights as they are
 Embedding:  token plus hashed-bigram row, then a norm;  a span of layers may run several times (own caches per pass)
 
+The Pobelorn design is the third member. Its layers are parallel blocks on the fp32 stream (RMS norm with a weight):
+
+Layer:      h = norm1(x); x <- x + mixer(h) + ff(h)                 (one norm, both sublayers read it)
+Mixers:     grouped-query attention whose queries and keys are rotated by position (interleaved pairs, stretched
+            frequencies) and then brought to unit RMS, behind a sliding window that keeps the first tokens, the values
+            mixed with those of the first such layer;  or linear attention with a fixed decay per head (fp32 state)
+ff:         squared-ReLU MLP, or routed gated experts (router with bias, softmax over the chosen logits) plus a
+            shared expert
+Embedding:  table row times a constant; the logits come from the same table
+
 The mechanisms are separate modules with their constants as constructor arguments (``WindowAttentionMixer``,
-``MLSTMMixer``, ``XieluMLP``, ``LatentAttentionMixer``, ``RoutedGLUExperts``); what they compute is documented with
+``MLSTMMixer``, ``XieluMLP``, ``LatentAttentionMixer``, ``RoutedGLUExperts``, ``RotaryWindowAttentionMixer``,
+``LightningMixer``, ``SquaredReluMLP``, ``RoutedSwiGLUExperts``); what they compute is documented with
 their kernels (``ops/window_attention.py``, ``ops/mlstm.py``, ``ops/post_norm.py``, ``ops/latent_attention.py``,
-``ops/sandwich.py``). The modules hold parameters and know how to run ONE step on the tensors of a
+``ops/sandwich.py``, ``ops/lightning.py``, ``ops/parallel_block.py``). The modules hold parameters and know how to run ONE step on the tensors of a
 batch plan; paged caches, state slots and the loop over layers belong to the model runner
 (``inference/model_runner.py::HybridModelRunner``).
 """
@@ -30,7 +41,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
+from ..ops import lightning as lightning_ops
 from ..ops import mlstm as mlstm_ops
+from ..ops import parallel_block as pblock
 from ..ops import latent_attention as lattn
 from ..ops import moe as moe_ops
 from ..ops import post_norm, sandwich, window_attention as wattn
@@ -46,14 +59,18 @@ class HybridConfig(ModelConfig):
     layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
     postln_alpha: float = 1.0
     design: str = "Kuzanex"
-    block_style: str = "post_norm"  # "post_norm": norm after every sum; "sandwich": norms before and after a sublayer
+    # "post_norm": norm after every sum; "sandwich": norms before and after a sublayer; "parallel": one norm, mixer and
+    # feed-forward read it and are added together
+    block_style: str = "post_norm"
+    embed_scale: float = 1.0  # factor on the embedding rows ("parallel" designs)
     loop: Optional[Dict[str, int]] = None  # layers start .. stop - 1 run `times` times in a row
     canon_taps: int = 0  # taps of the causal convolution on a mixer's input (0: none)
     bigram: Optional[Dict[str, int]] = None  # hashed-bigram embedding: buckets, mul_prev, mul_cur
 
     @property
     def has_recurrent_state(self) -> bool:
-        return any(l["type"] == "mlstm" for l in self.layers) or self.canon_taps > 1 or self.bigram is not None
+        return (any(l["type"] in ("mlstm", "lightning") for l in self.layers) or self.canon_taps > 1
+                or self.bigram is not None)
 
     @property
     def layer_runs(self) -> List[int]:
@@ -67,6 +84,8 @@ class HybridConfig(ModelConfig):
     def n_params(self, with_embedding: bool = True) -> int:
         if self.block_style == "sandwich":
             return self._n_params_sandwich(with_embedding)
+        if self.block_style == "parallel":
+            return self._n_params_parallel(with_embedding)
         W, n = self.hidden_size, 1
         for l in self.layers:
             m = l["mixer"]
@@ -96,7 +115,32 @@ class HybridConfig(ModelConfig):
             n += 2 * self.vocab_size * W + ((self.bigram["buckets"] + 1) * W if self.bigram else 0)
         return n
 
+    def _n_params_parallel(self, with_embedding: bool) -> int:
+        W = self.hidden_size
+        n = W  # final norm
+        for l in self.layers:
+            m = l["mixer"]
+            H, D, V = m["heads"], m["dim"], m["vdim"]
+            if l["type"] == "attention":
+                G = m["kv_heads"]
+                n += W * (H * D + G * D + G * V) + W * H * V + 1
+            else:
+                n += W * (2 * H * D + 2 * H * V) + H * V + W * H * V
+            n += W
+            e = l.get("mlp")
+            if e and e["kind"] == "dense":
+                n += 2 * W * e["ff"]
+            elif e:
+                n += e["router"]["experts"] * (W + 1 + 3 * W * e["expert"]["ff"])
+                if e.get("shared"):
+                    n += 3 * W * e["shared"]["ff"]
+        return n + (self.vocab_size * W if with_embedding else 0)
+
     def to_hf_dict(self) -> Dict[str, Any]:
+        if self.block_style == "parallel":
+            return {"architecture": self.design, "embedding": {"scale": self.embed_scale},
+                    "layers": json.loads(json.dumps(self.layers)), "norm": {"eps": self.rms_norm_eps},
+                    "vocab": self.vocab_size, "width": self.hidden_size}
         if self.block_style == "sandwich":
             d = {"architecture": self.design, "layers": [dict(l) for l in self.layers],
                  "norm": {"eps": self.rms_norm_eps}, "vocab": self.vocab_size, "width": self.hidden_size}
@@ -190,6 +234,43 @@ def lufivik_config_from_dir(path: str) -> HybridConfig:
         return lufivik_config(json.load(f))
 
 
+def pobelorn_config(d: Dict[str, Any]) -> HybridConfig:
+    """config.json of a Pobelorn checkpoint -> HybridConfig. Every size and constant is taken from it."""
+    layers = []
+    for i, l in enumerate(d["layers"]):
+        if l["type"] not in ("attention", "lightning"):
+            raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        mlp = l.get("mlp")
+        if mlp is not None and mlp.get("kind") not in ("dense", "moe"):
+            raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+        m = l["mixer"]
+        if l["type"] == "attention":
+            rot = m.get("rot")
+            if rot and (int(rot["dims"]) % 2 or int(rot["dims"]) > int(m["dim"])):
+                raise ValueError(f"layer {i}: the rotated part is an even number of at most dim coordinates")
+            if int(m["heads"]) % int(m.get("kv_heads", m["heads"])):
+                raise ValueError(f"layer {i}: heads is not a multiple of kv_heads")
+        elif len(m["decay"]) != int(m["heads"]):
+            raise ValueError(f"layer {i}: one decay per head is needed")
+        layers.append({"type": l["type"], "mixer": json.loads(json.dumps(m)),
+                       "mlp": json.loads(json.dumps(mlp)) if mlp is not None else None})
+    att = next((l["mixer"] for l in layers if l["type"] == "attention"), None)
+    widths = [(e["ff"] if e["kind"] == "dense" else e["expert"]["ff"]) for e in (l["mlp"] for l in layers) if e]
+    return HybridConfig(
+        family="pobelorn", design="Pobelorn", block_style="parallel", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), n_layers=len(layers), n_q_heads=int(att["heads"]) if att else 1,
+        n_kv_heads=int(att.get("kv_heads", att["heads"])) if att else 1, head_dim=int(att["dim"]) if att else 1,
+        intermediate_size=max(widths or [0]), rms_norm_eps=float(d["norm"]["eps"]),
+        max_position_embeddings=int(d.get("max_positions", 1 << 17)), tie_word_embeddings=True, qkv_bias=False,
+        pos_embed="none", layers=layers, embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+        eos_token_id=d.get("eos_token_id"), pad_token_id=d.get("pad_token_id"))
+
+
+def pobelorn_config_from_dir(path: str) -> HybridConfig:
+    with open(os.path.join(path, "config.json")) as f:
+        return pobelorn_config(json.load(f))
+
+
 class StepTensors:
     """What one batch plan hands to the mixers (all on the device): rows of the packed token batch (`cu_q`, longest
     row `max_q`), each row's context length after the step, cache slot of every token, page tables, position of each
@@ -201,6 +282,7 @@ class StepTensors:
         self.block_tables, self.first_pos, self.state_slots = block_tables, first_pos, state_slots
         self.nsplit, self.workspace = int(nsplit), workspace
         self.positions = positions  # position of every token (int32), for mixers that rotate by position
+        self.v_first = None  # this step's values of the first value-sharing attention layer [T, G Dv] (set by it)
 
 
 class WindowAttentionMixer(nn.Module):
@@ -352,6 +434,210 @@ class RoutedGLUExperts(nn.Module):
         return moe_ops.combine_rows_w32(grouped_gemm_rows(a, self.down, offsets), inv, topv)
 
 
+class RotaryWindowAttentionMixer(nn.Module):
+    """Grouped-query attention: queries and keys rotated by position on their first `rot_dims` coordinates (pairs of
+    neighbours, optionally stretched frequencies), then divided by their root mean square (no weight); scores times
+    `scale`; sliding window that keeps the first `keep_first` tokens; ordinary softmax. `v_mix` = "first": this
+    layer's values are what later layers mix in; "mix": v <- (1 - lam) v + lam v_first with the learned number `vmix`;
+    None: plain values. q | k | v are the first columns of the projection the block hands in."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, window: int, keep_first: int,
+                 rot: Optional[Dict[str, Any]], v_mix: Optional[str], eps: float, dtype, device):
+        super().__init__()
+        assert heads % kv_heads == 0 and v_mix in (None, "first", "mix")
+        self.H, self.G, self.D, self.V, self.eps = heads, kv_heads, dim, vdim, float(eps)
+        self.shape = wattn.ScoreShape(scale=float(scale), window=int(window), keep_first=int(keep_first))
+        self.rot = dict(rot) if rot else None
+        self.v_mix = v_mix
+        self.vmix = nn.Parameter(torch.zeros(1, dtype=dtype, device=device))  # read by "mix" layers only
+        self.table: Optional[torch.Tensor] = None
+
+    def in_rows(self) -> int:
+        return (self.H + self.G) * self.D + self.G * self.V
+
+    def out_cols(self) -> int:
+        return self.H * self.V
+
+    def cache_shape(self):
+        return self.G, self.D, self.V
+
+    def prepare(self, n_pos: int, tables: Dict[Any, torch.Tensor], device):
+        """The rotation table for positions below `n_pos`; mixers with the same constants share one."""
+        if not self.rot:
+            return
+        sc = self.rot.get("scaling") or None
+        key = ("rot", float(self.rot["base"]), int(self.rot["dims"]), int(n_pos),
+               tuple(sorted((k, float(v)) for k, v in sc.items())) if sc else None)
+        if key not in tables:
+            tables[key] = wattn.rotation_table(float(self.rot["base"]), int(self.rot["dims"]), int(n_pos), device, sc)
+        self.table = tables[key]
+
+    def step(self, proj: torch.Tensor, st: StepTensors, cache) -> torch.Tensor:
+        """proj [T, >= in_rows()] -> attended values [T, H Dv] (ahead of the output projection)."""
+        kc, vc = cache
+        H, G, D, V = self.H, self.G, self.D, self.V
+        vf = lam = None
+        if self.v_mix == "first":
+            st.v_first = proj[:, (H + G) * D:(H + G) * D + G * V]
+        elif self.v_mix == "mix":
+            vf, lam = st.v_first, self.vmix
+            assert vf is not None and vf.shape[1] == G * V, "the value-sharing layers need equal key/value head layouts"
+        q = wattn.rot_norm_cache_write(proj, st.positions, self.table, st.slots, kc, vc, H, self.eps, vf, lam)
+        o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
+                                   nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace)
+        return o.view(proj.shape[0], H * V)
+
+
+class LightningMixer(nn.Module):
+    """Linear attention with one fixed decay per head (``ops/lightning.py``): q | k | v | gate are the first columns
+    of the projection the block hands in, q, k and v pass through SiLU; the read-outs of all heads are RMS-normed
+    together (weight `norm`) and multiplied by sigmoid(gate)."""
+
+    def __init__(self, heads: int, dim: int, vdim: int, decay, eps: float, dtype, device):
+        super().__init__()
+        self.H, self.D, self.V, self.eps = heads, dim, vdim, float(eps)
+        self.register_buffer("decay", torch.tensor([float(x) for x in decay], dtype=torch.float32, device=device),
+                             persistent=False)
+        self.norm = nn.Parameter(torch.ones(heads * vdim, dtype=dtype, device=device))
+
+    def in_rows(self) -> int:
+        return 2 * self.H * self.D + 2 * self.H * self.V
+
+    def out_cols(self) -> int:
+        return self.H * self.V
+
+    def state_shape(self):
+        return self.H, self.D, self.V
+
+    def step(self, proj: torch.Tensor, st: StepTensors, state: torch.Tensor) -> torch.Tensor:
+        H, D, V = self.H, self.D, self.V
+        o = lightning_ops.lightning_scan(proj, 0, H * D, 2 * H * D, self.decay, st.cu_q, st.first_pos, st.state_slots,
+                                         state, max_q=st.max_q)
+        return lightning_ops.lightning_out(o, proj[:, 2 * H * D + H * V:2 * H * D + 2 * H * V], self.norm, self.eps)
+
+
+class SquaredReluMLP(nn.Module):
+    """down(max(up h, 0)^2). The up rows are part of the block's in-projection."""
+
+    def __init__(self, width: int, ff: int, dtype, device):
+        super().__init__()
+        self.ff = ff
+        self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype, device=device))
+
+    def in_rows(self) -> int:
+        return self.ff
+
+    def forward(self, cols: torch.Tensor, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
+        return F.linear(pblock.relu2_rows(cols), self.down)
+
+
+class RoutedSwiGLUExperts(nn.Module):
+    """Routed gated experts, down(silu(gate h) * (up h)), no biases: router logits W_r h + b in fp32 (on the fp32
+    normed input when the caller has it), the `top` largest are chosen and weighted by the softmax over the chosen
+    logits alone. Tokens are sorted by expert and every expert runs on a contiguous slab (grouped kernels, row ranges
+    on the device). A shared expert of the same form (`shared_ff` > 0) runs for every token and is added; its
+    gate | up rows are part of the block's in-projection."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int, dtype, device):
+        super().__init__()
+        assert 1 <= top <= experts
+        self.E, self.k, self.ff, self.shared_ff = experts, top, ff, int(shared_ff)
+        self.router = nn.Parameter(torch.empty(experts, width, dtype=dtype, device=device))
+        self.router_bias = nn.Parameter(torch.zeros(experts, dtype=dtype, device=device))
+        self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width, dtype=dtype, device=device))
+        self.down = nn.Parameter(torch.empty(experts, width, ff, dtype=dtype, device=device))
+        self.shared_down = (nn.Parameter(torch.empty(width, shared_ff, dtype=dtype, device=device))
+                            if shared_ff > 0 else None)
+
+    def in_rows(self) -> int:
+        return 2 * self.shared_ff
+
+    def forward(self, cols: torch.Tensor, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
+        if hc.dtype == torch.float32:
+            z = F.linear(hc, self.router, self.router_bias)
+        else:  # fp32 products on the norm's fp32 output when there is one, else on its rounding
+            z = F.linear(h32 if h32 is not None else hc.float(), self.router.float(), self.router_bias.float())
+        # softmax over all logits, the k largest re-normalised: the softmax over the chosen logits
+        topv, topi = moe_ops.moe_topk(z, self.k, True, out_dtype=torch.float32)
+        order, inv, src_row, offsets = moe_ops.moe_sort(topi.reshape(-1), self.E, self.k)
+        xs = moe_ops._gather_rows(hc, src_row)
+        a = pblock.glu_rows(grouped_gemm_rows(xs, self.gate_up, offsets))
+        y = moe_ops.combine_rows_w32(grouped_gemm_rows(a, self.down, offsets), inv, topv)
+        if self.shared_down is not None:
+            y = torch.addmm(y, pblock.glu_rows(cols), self.shared_down.t())
+        return y
+
+
+class ParallelBlock(nn.Module):
+    """A layer whose mixer and feed-forward read the same norm of the stream: ONE projection of the normed input
+    yields the mixer's operands and the feed-forward's dense first stage (up rows, or the shared expert's gate | up),
+    side by side; the two outputs are returned separately and summed into the stream by the caller's closing kernel."""
+
+    def __init__(self, cfg: HybridConfig, spec: Dict[str, Any], v_mix: Optional[str], dtype, device):
+        super().__init__()
+        W, m, eps = cfg.hidden_size, spec["mixer"], cfg.rms_norm_eps
+        self.kind = spec["type"]
+        if self.kind == "attention":
+            mask = m.get("mask") or {}
+            self.mix = RotaryWindowAttentionMixer(
+                int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m.get("scale", float(m["dim"]) ** -0.5)), int(mask.get("size") or 0),
+                int(mask.get("keep_first") or 0), m.get("rot"), v_mix, eps, dtype, device)
+        else:
+            self.mix = LightningMixer(int(m["heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])), m["decay"], eps,
+                                      dtype, device)
+        e = spec.get("mlp")
+        if not e:
+            self.mlp = None
+        elif e["kind"] == "dense":
+            self.mlp = SquaredReluMLP(W, int(e["ff"]), dtype, device)
+        else:
+            self.mlp = RoutedSwiGLUExperts(W, int(e["expert"]["ff"]), int(e["router"]["experts"]),
+                                           int(e["router"]["top"]), int((e.get("shared") or {}).get("ff", 0)), dtype,
+                                           device)
+        self.norm1 = nn.Parameter(torch.ones(W, dtype=dtype, device=device))
+        self.n_mix = self.mix.in_rows()
+        self.w_in = nn.Parameter(torch.empty(self.n_mix + (self.mlp.in_rows() if self.mlp is not None else 0), W,
+                                             dtype=dtype, device=device))
+        self.o = nn.Parameter(torch.empty(W, self.mix.out_cols(), dtype=dtype, device=device))
+        self.needs32 = isinstance(self.mlp, RoutedSwiGLUExperts)  # the router reads the norm's fp32 output
+
+    def step(self, hc: torch.Tensor, h32: Optional[torch.Tensor], st: StepTensors, cache, state):
+        """(hc, h32) = norm1 of the stream in the compute dtype and (when asked for) fp32 -> (mixer output, feed-forward
+        output or None), both [T, W] in the compute dtype."""
+        proj = F.linear(hc, self.w_in)
+        y = F.linear(self.mix.step(proj, st, cache if self.kind == "attention" else state), self.o)
+        if self.mlp is None:
+            return y, None
+        return y, self.mlp(proj[:, self.n_mix:], hc, h32)
+
+    def checkpoint_tensors(self, p: str) -> Dict[str, torch.Tensor]:
+        m, w = self.mix, self.w_in.data
+        out = {p + "norm1": self.norm1.data, p + "mix.o": self.o.data}
+        if self.kind == "attention":
+            a, b = m.H * m.D, (m.H + m.G) * m.D
+            out.update({p + "mix.q": w[:a], p + "mix.k": w[a:b], p + "mix.v": w[b:self.n_mix]})
+            out[p + "mix.vmix"] = m.vmix.data.view(())
+        else:
+            a, b, c = m.H * m.D, 2 * m.H * m.D, 2 * m.H * m.D + m.H * m.V
+            out.update({p + "mix.q": w[:a], p + "mix.k": w[a:b], p + "mix.v": w[b:c], p + "mix.g": w[c:self.n_mix],
+                        p + "mix.norm": m.norm.data})
+        e, q = self.mlp, p + "mlp."
+        if isinstance(e, SquaredReluMLP):
+            out[q + "up"], out[q + "down"] = w[self.n_mix:], e.down.data
+        elif e is not None:
+            out[q + "router"], out[q + "router.b"] = e.router.data, e.router_bias.data
+            for i in range(e.E):
+                out[q + f"e{i}.gate"] = e.gate_up.data[i, :e.ff]
+                out[q + f"e{i}.up"] = e.gate_up.data[i, e.ff:]
+                out[q + f"e{i}.down"] = e.down.data[i]
+            if e.shared_down is not None:
+                sf = e.shared_ff
+                out[q + "shared.gate"], out[q + "shared.up"] = w[self.n_mix:self.n_mix + sf], w[self.n_mix + sf:]
+                out[q + "shared.down"] = e.shared_down.data
+        return out
+
+
 class SandwichBlock(nn.Module):
     """A layer whose sublayers sit between two layer norms, with a sigmoid gate computed from the sublayer's normed
     input, one scale per channel on the result, and a causal convolution on what the mixer reads."""
@@ -474,8 +760,18 @@ class HybridDecoder(nn.Module):
         self.vocab_range = (0, cfg.vocab_size)
         self.embed = nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device))
         self.sandwich = cfg.block_style == "sandwich"
+        self.parallel = cfg.block_style == "parallel"
         self.layer_runs = cfg.layer_runs
-        if self.sandwich:
+        if self.parallel:
+            blocks, seen_first = [], False
+            for spec in cfg.layers:
+                v_mix = None
+                if spec["type"] == "attention" and spec["mixer"].get("v_mix"):
+                    v_mix, seen_first = ("mix" if seen_first else "first"), True
+                blocks.append(ParallelBlock(cfg, spec, v_mix, dtype, device))
+            self.layers = nn.ModuleList(blocks)
+            self.norm = nn.Parameter(torch.ones(cfg.hidden_size, dtype=dtype, device=device))
+        elif self.sandwich:
             W = cfg.hidden_size
             self.bigram = (nn.Parameter(torch.empty(cfg.bigram["buckets"] + 1, W, dtype=dtype, device=device))
                            if cfg.bigram else None)
@@ -487,13 +783,15 @@ class HybridDecoder(nn.Module):
         else:
             self.layers = nn.ModuleList([HybridBlock(cfg, spec, dtype, device) for spec in cfg.layers])
             self.norm = nn.Parameter(torch.ones(1, dtype=dtype, device=device))
-        self.head = nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device))
+        # designs whose logits come from the embedding table have no second matrix
+        self.head = (None if cfg.tie_word_embeddings else
+                     nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device)))
         self.flat: Optional[FlatParams] = None
         self.flat_experts = None
 
     @property
     def head_weight(self) -> torch.Tensor:
-        return self.head
+        return self.head if self.head is not None else self.embed
 
     def flatten(self, pad_to: int = 1, expert_pad_to=None) -> FlatParams:
         self.flat = FlatParams(self, self.dtype, next(self.parameters()).device, pad_to)
@@ -504,7 +802,18 @@ class HybridDecoder(nn.Module):
         W = self.cfg.hidden_size
         for n, p in self.named_parameters():
             leaf = n.rsplit(".", 1)[-1]
-            if self.sandwich and leaf != "embed" and (p.dim() == 1 or leaf == "canon1"):
+            if self.parallel:
+                if leaf == "vmix":
+                    p.data.copy_(0.2 + 0.6 * torch.rand(p.shape, generator=g))
+                elif leaf == "router_bias":
+                    p.data.copy_(0.5 * torch.randn(p.shape, generator=g))
+                elif p.dim() == 1:  # norm weights
+                    p.data.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+                elif leaf == "embed":  # rows of about unit RMS once the embedding's factor is applied
+                    p.data.copy_(torch.randn(p.shape, generator=g) / max(self.cfg.embed_scale, 1e-6))
+                else:
+                    p.data.copy_(torch.randn(p.shape, generator=g) / (p.shape[-1] ** 0.5))
+            elif self.sandwich and leaf != "embed" and (p.dim() == 1 or leaf == "canon1"):
                 if leaf.endswith("_bias"):
                     p.data.copy_(0.1 * torch.randn(p.shape, generator=g))
                 elif leaf == "canon1":
@@ -544,6 +853,11 @@ class HybridDecoder(nn.Module):
     # ------------------------------------------------------------------------- checkpoint names
     def checkpoint_tensors(self) -> Dict[str, torch.Tensor]:
         """Checkpoint name -> the view of this model's parameters that holds it (fused projections are sliced)."""
+        if self.parallel:
+            out = {"embed": self.embed.data, "final.norm": self.norm.data}
+            for i, blk in enumerate(self.layers):
+                out.update(blk.checkpoint_tensors(f"l{i}."))
+            return out
         if self.sandwich:
             out = {"embed": self.embed.data, "head": self.head.data, "final.norm": self.norm.data,
                    "final.norm.b": self.norm_bias.data, "embed.norm": self.embed_norm.data,
@@ -586,6 +900,13 @@ class HybridDecoder(nn.Module):
                 out[q + "act"] = blk.mlp.act.data
         return out
 
+    def checkpoint_optional(self) -> set:
+        """Names a checkpoint may leave out: numbers that this model's layers never read."""
+        if not self.parallel:
+            return set()
+        return {f"l{i}.mix.vmix" for i, blk in enumerate(self.layers)
+                if blk.kind == "attention" and blk.mix.v_mix != "mix"}
+
     def assign_named_tensors(self, tensors: Dict[str, torch.Tensor], strict: bool = True):
         views = self.checkpoint_tensors()
         unknown = [n for n in tensors if n not in views]
@@ -610,7 +931,7 @@ class HybridDecoder(nn.Module):
                 names = list(f.keys())
                 self.assign_named_tensors({k: f.get_tensor(k) for k in names}, strict=strict)
                 seen.update(names)
-        missing = sorted(set(self.checkpoint_tensors()) - seen)
+        missing = sorted(set(self.checkpoint_tensors()) - seen - self.checkpoint_optional())
         if strict and missing:
             raise KeyError(f"checkpoint lacks {len(missing)} tensor(s): {missing[:8]}")
 

@@ -1,5 +1,8 @@
 """Sliding-window attention over the paged cache with shaped scores: soft cap, linear distance bias, mixing of the
-heads' scores ahead of the softmax, an optional value-less sink in the denominator.
+heads' scores ahead of the softmax, an optional value-less sink in the denominator, optionally the first tokens of a
+sequence kept visible beyond the window. Two ways of preparing queries and keys: RMS norm with a weight
+(`qk_norm_cache_write`), or rotation by position followed by a weightless RMS norm, with the values optionally mixed
+with those of another layer (`rot_norm_cache_write`).
 
 GPU: ``csrc/hip/window_attn.hip`` (one kernel for prompt portions and, with a split key range, for decoding).
 CPU: a PyTorch formulation used by the unit tests and CPU runs.
@@ -24,6 +27,7 @@ class ScoreShape:
     slope_exp: float = 0.0  # slope of head h: 2^(-slope_exp (h + 1) / H); 0: no distance bias
     window: int = 0  # <= 0: all earlier tokens
     sink: bool = False
+    keep_first: int = 0  # keys at positions below this stay visible to every later query, whatever the window
 
 
 def alloc_window_cache(num_pages: int, n_kv_heads: int, k_dim: int, v_dim: int, dtype, device
@@ -66,10 +70,86 @@ def qk_norm_cache_write(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_
     return q
 
 
-def decode_splits(batch: int, window: int, max_context: int) -> int:
+def rotation_table(base: float, dims: int, n_pos: int, device, scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp32 [n_pos, dims]: m cos(p f_i) for i < dims/2, then m sin(p f_i), with f_i = base^(-2i/dims).
+
+    `scaling` = {factor, original, fast, slow} stretches the slow pairs for contexts beyond `original` positions (YaRN:
+    Peng et al., "YaRN: Efficient Context Window Extension of Large Language Models"): with
+    d(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the frequency is f_i (1 - ramp_i) + f_i ramp_i / factor, and
+    m = 0.1 ln(factor) + 1 (1 without scaling). Angles are formed in float64 and rounded once."""
+    assert dims % 2 == 0 and dims > 0
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    m = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def d_of(turns: float) -> float:
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+        lo = max(math.floor(d_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(d_of(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        m = 0.1 * math.log(factor) + 1.0
+    a = torch.arange(n_pos, dtype=torch.float64).unsqueeze(1) * f
+    return (torch.cat([a.cos(), a.sin()], 1) * m).float().to(device)
+
+
+def rot_norm_cache_write(proj: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
+                         slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, n_heads: int, eps: float,
+                         v_first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """proj [T, >= (H + G) D + G Dv]: q heads | k heads | v heads (more columns may follow). Rotates the first
+    table.shape[1] coordinates of every q and k head at the token's position (pairs (2i, 2i + 1); `table` as
+    `rotation_table` makes it, None: no rotation), divides every head by its root mean square over D, and writes k and
+    v of tokens with slot >= 0 into the paged caches; with `v_first` [T, G Dv] (a view with unit column stride) and
+    `lam` (one number) the values become (1 - lam) v + lam v_first first. Returns the queries [T, H, D]."""
+    T = proj.shape[0]
+    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[3]
+    H = n_heads
+    R = 0 if table is None else table.shape[1]
+    assert proj.stride(1) == 1 and proj.shape[1] >= (H + G) * D + G * V and R <= D and R % 2 == 0
+    assert (v_first is None) == (lam is None)
+    q = torch.empty(T, H, D, dtype=proj.dtype, device=proj.device)
+    if L.use_hip(proj):
+        assert slots.dtype == torch.int64 and kcache.dtype == proj.dtype and positions.dtype == torch.int32
+        assert table is None or (table.dtype == torch.float32 and table.is_contiguous())
+        assert v_first is None or (v_first.dtype == proj.dtype and v_first.stride(1) == 1
+                                   and v_first.shape == (T, G * V) and lam.dtype == proj.dtype and lam.numel() == 1)
+        if table is None:  # one row of angle zero
+            table = torch.zeros(1, 0, dtype=torch.float32, device=proj.device)
+        L.check(L.lib().areal_rot_norm_cache_write(
+            L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(positions), L.ptr(table), L.c_int(table.shape[0]), L.c_int(R),
+            L.ptr(slots), L.ptr(v_first), L.c_int64(v_first.stride(0) if v_first is not None else 0), L.ptr(lam),
+            L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V),
+            L.c_float(eps), L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "rot_norm_cache_write")
+        return q
+    qk = proj[:, :(H + G) * D].float().view(T, H + G, D)
+    if R:
+        cs = table[positions.long()]
+        c, s = cs[:, :R // 2].unsqueeze(1), cs[:, R // 2:].unsqueeze(1)
+        u, w = qk[..., 0:R:2], qk[..., 1:R:2]
+        rot = torch.stack([u * c - w * s, w * c + u * s], -1).reshape(T, H + G, R)
+        qk = torch.cat([rot, qk[..., R:]], -1)
+    qk = qk * torch.rsqrt(qk.pow(2).mean(-1, keepdim=True) + eps)
+    q.copy_(qk[:, :H])
+    v = proj[:, (H + G) * D:(H + G) * D + G * V].float()
+    if v_first is not None:
+        lam_f = lam.float().reshape(())
+        v = (1.0 - lam_f) * v + lam_f * v_first.float()
+    ok = slots >= 0
+    if ok.any():
+        pg, off = (slots[ok] // PAGE_SIZE).long(), (slots[ok] % PAGE_SIZE).long()
+        kcache[pg, :, off, :] = qk[:, H:][ok].to(kcache.dtype)
+        vcache[pg, :, off, :] = v[ok].view(-1, G, V).to(vcache.dtype)
+    return q
+
+
+def decode_splits(batch: int, window: int, max_context: int, keep_first: int = 0) -> int:
     """Key-range splits of a decode launch: about two workgroups per compute unit, down to one page each (a
     workgroup walks its pages one after the other, so short ranges are what makes a decode step short)."""
-    span = max_context if window <= 0 else min(window + PAGE_SIZE, max_context)
+    span = max_context if window <= 0 else min(window + PAGE_SIZE + max(0, keep_first), max_context)
     pages = max(1, (span + PAGE_SIZE - 1) // PAGE_SIZE)
     return int(max(1, min(512 // max(1, batch), pages, 32)))
 
@@ -112,7 +192,8 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
             L.ptr(ctx_len), L.ptr(mix), L.ptr(gate), L.c_int64(gate.stride(0) if gate is not None else 0), L.ptr(out),
             L.ptr(pa), L.ptr(pm), L.c_int(B), L.c_int(int(max_q)), L.c_int(T),
             L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_int(bq), L.c_float(shape.scale),
-            L.c_float(shape.softcap), L.c_float(shape.slope_exp), L.c_int(int(shape.window)), L.c_int(int(shape.sink)),
+            L.c_float(shape.softcap), L.c_float(shape.slope_exp), L.c_int(int(shape.window)),
+            L.c_int(int(shape.keep_first)), L.c_int(int(shape.sink)),
             L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.c_int(int(matrix_cores)), L.stream_ptr()), "window_attn")
         return out
     out = torch.zeros(T, H, V, dtype=torch.float32, device=q.device)
@@ -124,7 +205,7 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         n, ctx = cq[b + 1] - cq[b], cl[b]
         if n == 0:
             continue
-        lo = 0 if shape.window <= 0 else max(0, ctx - n - shape.window + 1)
+        lo = 0 if (shape.window <= 0 or shape.keep_first > 0) else max(0, ctx - n - shape.window + 1)
         pages = block_tables[b, :(ctx + PAGE_SIZE - 1) // PAGE_SIZE].long()
         kk = kcache[pages].permute(1, 0, 2, 3).reshape(G, -1, D)[:, lo:ctx].float().repeat_interleave(rep, 0)
         vv = vcache[pages].permute(1, 0, 2, 3).reshape(G, -1, V)[:, lo:ctx].float().repeat_interleave(rep, 0)
@@ -136,7 +217,7 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         s = s - slopes.view(H, 1, 1) * (i - j).float()
         if mix is not None:
             s = torch.einsum("hg,gij->hij", mix.float(), s)
-        ok = (i - j >= 0) & ((i - j < shape.window) if shape.window > 0 else True)
+        ok = (i - j >= 0) & (((i - j < shape.window) | (j < shape.keep_first)) if shape.window > 0 else True)
         s = s.masked_fill(~ok, float("-inf"))
         m = s.max(-1, keepdim=True).values
         if shape.sink:

@@ -4,7 +4,8 @@
 //   s_g       <- cap * tanh(s_g / cap)                             (cap > 0; otherwise left as it is)
 //   s_g       <- s_g - slope_g * (i - j),  slope_g = 2^(-slope_exp * (g + 1) / H)     (slope_exp = 0: no bias)
 //   t_h        = sum_g M[h, g] s_g                                 head mixing (M = null: t_h = s_h)
-//   visible:     0 <= i - j < window                               (window <= 0: every earlier key)
+//   visible:     0 <= i - j < window, or j <= i and j < keep_first    (window <= 0: every earlier key; the first
+//                keep_first tokens of a sequence stay visible to every later query, at their true positions)
 //   p_h(j)     = exp(t_h(j)) / (sink + sum_j' exp(t_h(j')))        sink = 1: a key of score 0 that has no value
 //   o_h(i)     = sum_j p_h(j) v_c(h)(j)  [* sigmoid(gate_h(i)) when a gate is given: one number per head and token]
 //
@@ -72,6 +73,67 @@ __global__ void __launch_bounds__(256) qk_norm_cache_write_kernel(
   }
 }
 
+// Per token: rotate the first R coordinates of every query and key head by the token's position (neighbouring
+// coordinates (2i, 2i + 1) form a pair; table rows hold R / 2 cosines, then R / 2 sines, already multiplied by
+// whatever factor the rotation carries), then divide the head by its root mean square over D (no weight). Queries go
+// to q_out, keys into the K cache. Values: v <- (1 - lam) v + lam v_first when `v_first` is given (rows of G V values of
+// the same tokens, from the layer whose values are shared), then into the V cache.
+template <typename T>
+__global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
+    const T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ table,
+    int n_pos, int R, const int64_t* __restrict__ slots, const T* __restrict__ v_first, int64_t vf_stride,
+    const T* __restrict__ lam_p, T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache, int H, int G,
+    int D, int V, float eps) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * row_stride;
+  const int64_t slot = slots[t];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t page = slot >= 0 ? (size_t)(slot / PAGE) : 0;
+  const int off = slot >= 0 ? (int)(slot % PAGE) : 0;
+  const int pos = min(max(positions[t], 0), n_pos - 1);
+  const float* cs = table + (size_t)pos * R;
+  const int half = R / 2;
+  for (int u = wave; u < H + G; u += 4) {
+    if (u >= H && slot < 0) continue;
+    const T* src = row + (size_t)u * D;
+    T* dst = u < H ? q_out + ((size_t)t * H + u) * D : kcache + ((page * G + (u - H)) * PAGE + off) * D;
+    // units of work: pairs below R, single coordinates from R on
+    const int units = half + (D - R);
+    float ss = 0.f;
+    for (int i = lane; i < units; i += 64) {
+      if (i < half) {
+        const float a = ldf<T>(src, 2 * i), b = ldf<T>(src, 2 * i + 1), c = cs[i], s = cs[half + i];
+        const float x = a * c - b * s, y = b * c + a * s;
+        ss += x * x + y * y;
+      } else {
+        const float x = ldf<T>(src, R + i - half);
+        ss += x * x;
+      }
+    }
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / (float)D + eps);
+    for (int i = lane; i < units; i += 64) {
+      if (i < half) {
+        const float a = ldf<T>(src, 2 * i), b = ldf<T>(src, 2 * i + 1), c = cs[i], s = cs[half + i];
+        stf<T>(dst, 2 * i, (a * c - b * s) * r);
+        stf<T>(dst, 2 * i + 1, (b * c + a * s) * r);
+      } else {
+        stf<T>(dst, R + i - half, ldf<T>(src, R + i - half) * r);
+      }
+    }
+  }
+  if (slot >= 0) {
+    const T* vsrc = row + (size_t)(H + G) * D;
+    const float lam = v_first ? ldf<T>(lam_p, 0) : 0.f;
+    for (int i = threadIdx.x; i < G * V; i += 256) {
+      const int c = i / V, v = i % V;
+      float x = ldf<T>(vsrc, i);
+      if (v_first) x = (1.f - lam) * x + lam * ldf<T>(v_first, (size_t)t * vf_stride + i);
+      stf<T>(vcache, ((page * G + c) * PAGE + off) * V + v, x);
+    }
+  }
+}
+
 struct AttnShape {
   int H, G, D, V, BQ;
   // LDS layout in floats
@@ -87,7 +149,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     const T* __restrict__ q, const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const T* __restrict__ mix, const T* __restrict__ gate, int64_t gate_stride,
-    T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int sink,
+    T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int keep, int sink,
     int nsplit) {
   extern __shared__ float lds[];
   const int H = sh.H, G = sh.G, D = sh.D, V = sh.V, BQ = sh.BQ;
@@ -123,14 +185,18 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
   if (mix)
     for (int i = tid; i < H * H; i += 256) mixs[i] = ldf<T>(mix, i);
 
-  // visible keys of the tile: [j_lo, j_hi); pages [p_lo, p_hi), this split's share of them
+  // visible keys of the tile: [j_lo, j_hi) and the kept first ones; pages [0, p_keep) and [p_lo, p_hi), this split's
+  // share of them
   const int j_hi = pos0 + nq;
   const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
-  const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
-  const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
+  const int p_keep = min((max(keep, 0) + PAGE - 1) / PAGE, p_lo);
+  const int n_pages = p_keep + p_hi - p_lo;
+  const int per = (n_pages + nsplit - 1) / nsplit;
+  const int my_lo = split * per, my_hi = min(n_pages, my_lo + per);
 
-  for (int pg = my_lo; pg < my_hi; ++pg) {
+  for (int pi = my_lo; pi < my_hi; ++pi) {
+    const int pg = pi < p_keep ? pi : p_lo + pi - p_keep;
     const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
     const int jb = pg * PAGE;
     // ---- shaped scores of every head
@@ -172,7 +238,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
         s = S1[e];
       }
       const int dist = pos0 + qi - (jb + kj);
-      const bool ok = qi < nq && dist >= 0 && (window <= 0 || dist < window);
+      const bool ok = qi < nq && dist >= 0 && (window <= 0 || dist < window || jb + kj < keep);
       S2[e] = ok ? s : -INFINITY;
     }
     __syncthreads();
@@ -258,7 +324,7 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const bf16_t* __restrict__ mix, const bf16_t* __restrict__ gate,
     int64_t gate_stride, bf16_t* __restrict__ out, int H, int G, float scale, float softcap, float slope_exp,
-    int window, int sink) {
+    int window, int keep, int sink) {
   constexpr int D = DK * 32, V = VT_ * 16, KS = D + 8, VS = PAGE + 8, SS = PAGE + 4;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   unsigned* SM = reinterpret_cast<unsigned*>(smem);                      // [16][16][SS] 4-byte slots
@@ -301,9 +367,11 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
   const int j_hi = pos0 + nq;
   const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+  const int p_keep = min((max(keep, 0) + PAGE - 1) / PAGE, p_lo);  // pages of kept first tokens below the window's
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
 
-  for (int pg = p_lo; pg < p_hi; ++pg) {
+  for (int pi = 0; pi < p_keep + p_hi - p_lo; ++pi) {
+    const int pg = pi < p_keep ? pi : p_lo + pi - p_keep;
     const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
     const int jb = pg * PAGE;
     __syncthreads();  // the page before is consumed (first time: the set-up above is visible)
@@ -359,8 +427,8 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
         m1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b1, m1, 0, 0, 0);
       }
       const int d0 = pos0 + qi - (jb + r16), d1 = d0 - 16;
-      const bool ok0 = qi < nq && d0 >= 0 && (window <= 0 || d0 < window);
-      const bool ok1 = qi < nq && d1 >= 0 && (window <= 0 || d1 < window);
+      const bool ok0 = qi < nq && d0 >= 0 && (window <= 0 || d0 < window || jb + r16 < keep);
+      const bool ok1 = qi < nq && d1 >= 0 && (window <= 0 || d1 < window || jb + 16 + r16 < keep);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int h = 4 * quad + i;
@@ -435,7 +503,7 @@ size_t mfma_lds_bytes(int G, int D, int V) {
 }
 int mfma_heads_per_wave(int H) { return (H % 4 == 0 && H >= 16) ? 4 : ((H % 2 == 0 && H >= 8) ? 2 : 1); }
 bool mfma_usable(int H, int G, int D, int V) {
-  if (H > 16 || H < 1 || G < 1 || H % G != 0 || (D != 64 && D != 128) || (V != 64 && V != 128)) return false;
+  if (H > 16 || H < 1 || G < 1 || H % G != 0 || (D != 64 && D != 128) || (V != 32 && V != 64 && V != 128)) return false;
   if (H / mfma_heads_per_wave(H) > 8) return false;
   return mfma_lds_bytes(G, D, V) <= 160 * 1024;
 }
@@ -444,7 +512,7 @@ template <int HPW, int MAXT>
 int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* kc, const bf16_t* vc,
                 const int* bt, int max_pages, const int* cu_q, const int* ctx_len, const bf16_t* mix,
                 const bf16_t* gate, int64_t gate_stride, bf16_t* out, int H, int G, int D, int V, float scale,
-                float softcap, float slope_exp, int window, int sink) {
+                float softcap, float slope_exp, int window, int keep, int sink) {
 #define MFMA_CASE(DKV, VTV)                                                                                        \
   do {                                                                                                             \
     static bool raised = false; /* once per kernel: no attribute call inside a stream capture later */            \
@@ -455,10 +523,12 @@ int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q
     }                                                                                                              \
     hipLaunchKernelGGL((window_attn_mfma_kernel<HPW, DKV, VTV, MAXT>), grid, dim3(nthr), lds, st, q, kc, vc, bt,   \
                        max_pages, cu_q, ctx_len, mix, gate, gate_stride, out, H, G, scale, softcap, slope_exp,     \
-                       window, sink);                                                                              \
+                       window, keep, sink);                                                                        \
   } while (0)
-  if (D == 64 && V == 64) MFMA_CASE(2, 4);
+  if (D == 64 && V == 32) MFMA_CASE(2, 2);
+  else if (D == 64 && V == 64) MFMA_CASE(2, 4);
   else if (D == 64 && V == 128) MFMA_CASE(2, 8);
+  else if (D == 128 && V == 32) MFMA_CASE(4, 2);
   else if (D == 128 && V == 64) MFMA_CASE(4, 4);
   else MFMA_CASE(4, 8);
 #undef MFMA_CASE
@@ -505,6 +575,24 @@ extern "C" int areal_qk_norm_cache_write(const void* proj, int64_t row_stride, c
   return (int)hipGetLastError();
 }
 
+// proj rows: q heads | k heads | v heads from the pointer on. table fp32 [n_pos, R]; v_first / lam null: values as they are.
+extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, const int* positions, const float* table,
+                                          int n_pos, int R, const int64_t* slots, const void* v_first, int64_t vf_stride,
+                                          const void* lam, void* q_out, void* kcache, void* vcache, int T, int H, int G,
+                                          int D, int V, float eps, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  if (R < 0 || R > D || R % 2 != 0 || n_pos < 1 || (v_first && !lam)) return -1;
+  if (dt == 0)
+    hipLaunchKernelGGL(rot_norm_cache_write_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
+                       positions, table, n_pos, R, slots, (const bf16_t*)v_first, vf_stride, (const bf16_t*)lam,
+                       (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps);
+  else
+    hipLaunchKernelGGL(rot_norm_cache_write_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
+                       positions, table, n_pos, R, slots, (const float*)v_first, vf_stride, (const float*)lam,
+                       (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps);
+  return (int)hipGetLastError();
+}
+
 // Largest query tile (16, 8, 4, 2, 1) whose LDS footprint fits the workgroup limit; 0 if even one query does not.
 extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
   for (int bq = want; bq >= 1; bq >>= 1) {
@@ -519,8 +607,8 @@ extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
 extern "C" int areal_window_attn(const void* q, const void* kcache, const void* vcache, const int* block_tables,
                                  int max_pages, const int* cu_q, const int* ctx_len, const void* mix, const void* gate,
                                  int64_t gate_stride, void* out, float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
-                                 int bq, float scale, float softcap, float slope_exp, int window, int sink, int nsplit,
-                                 int dt, int matrix_cores, hipStream_t st) {
+                                 int bq, float scale, float softcap, float slope_exp, int window, int keep, int sink,
+                                 int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1) return -1;
   if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(H, G, D, V)) {
@@ -530,7 +618,7 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
 #define MFMA_ARGS                                                                                                  \
   mgrid, nthr, mlds, st, (const bf16_t*)q, (const bf16_t*)kcache, (const bf16_t*)vcache, block_tables, max_pages,   \
       cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, G, D, V, scale, softcap, \
-      slope_exp, window, sink
+      slope_exp, window, keep, sink
     if (hpw == 4) return launch_mfma<4, 256>(MFMA_ARGS);
     if (hpw == 2) return launch_mfma<2, 512>(MFMA_ARGS);
     return launch_mfma<1, 512>(MFMA_ARGS);
@@ -551,7 +639,8 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
     }                                                                                                                \
     hipLaunchKernelGGL(window_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)kcache,            \
                        (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (const TT*)gate,   \
-                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit); \
+                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, softcap, slope_exp, window, keep, sink,   \
+                       nsplit);                                                                                     \
     if (nsplit > 1)                                                                                                  \
       hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,           \
                          (const TT*)gate, gate_stride, (TT*)out, H, V, nsplit);                                      \
