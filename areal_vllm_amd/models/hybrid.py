@@ -769,6 +769,10 @@ class HybridDecoder(nn.Module):
                 if spec["type"] == "attention" and spec["mixer"].get("v_mix"):
                     v_mix, seen_first = ("mix" if seen_first else "first"), True
                 blocks.append(ParallelBlock(cfg, spec, v_mix, dtype, device))
+                if v_mix == "mix":
+                    first = next(b.mix for b in blocks if b.kind == "attention" and b.mix.v_mix == "first")
+                    if (first.G, first.V) != (blocks[-1].mix.G, blocks[-1].mix.V):
+                        raise ValueError("layers that mix values need the key/value heads and value size of the first")
             self.layers = nn.ModuleList(blocks)
             self.norm = nn.Parameter(torch.ones(cfg.hidden_size, dtype=dtype, device=device))
         elif self.sandwich:

@@ -166,3 +166,12 @@ def forward(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int]) -> T
         streams.append(x.clone())
     logits = (rms(x, eps) * weights["final.norm"].to(F64)) @ E.T
     return logits, streams
+
+
+def greedy(cfg: Dict, weights: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        logits, _ = forward(cfg, weights, toks)
+        out.append(int(torch.argmax(logits[-1])))
+        toks.append(out[-1])
+    return out

@@ -1,0 +1,621 @@
+"""Pobelorn (layer-list decoder of parallel blocks: window attention on rotated, unit-RMS queries and keys that keeps
+the first tokens and mixes values across layers; lightning attention with a decay per head; squared-ReLU and routed +
+shared gated feed-forward) against the plain float64 formulation in ``pobelorn_oracle.py``: every mechanism alone,
+then the serving engine - scheduler, paged caches, state slots, prefill and decode plans - on small random models of
+several shapes. Every test runs on the CPU formulations of the ops and, marked `gpu`, on the HIP kernels."""
+import math
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import pobelorn_oracle as O  # noqa: E402
+
+from areal_vllm_amd.api.cli_args import InferenceServerConfig  # noqa: E402
+from areal_vllm_amd.inference.engine import NativeInferenceEngine  # noqa: E402
+from areal_vllm_amd.models.config import ModelConfig  # noqa: E402
+from areal_vllm_amd.models.hybrid import RoutedSwiGLUExperts  # noqa: E402
+from areal_vllm_amd.ops import lightning as lightning_ops  # noqa: E402
+from areal_vllm_amd.ops import parallel_block as pb  # noqa: E402
+from areal_vllm_amd.ops import window_attention as wattn  # noqa: E402
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+CASES = [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu),
+         pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu)]
+OP_CASES = [("cpu", torch.float32), ("cpu", torch.bfloat16),
+            pytest.param("cuda", torch.float32, marks=pytest.mark.gpu),
+            pytest.param("cuda", torch.bfloat16, marks=pytest.mark.gpu)]
+F64 = torch.float64
+PAGE = 32
+
+
+def tol(dtype):
+    return 2e-4 if dtype in ("float32", torch.float32) else 6e-2
+
+
+def row_errors(got, want):
+    got, want = torch.as_tensor(got).to(F64), torch.as_tensor(want).to(F64)
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    ref = (want - want.mean(-1, keepdim=True)).pow(2).mean(-1).sqrt().clamp(min=1e-9)
+    return d.pow(2).mean(-1).sqrt() / ref
+
+
+def rel_err(got, want):
+    """Per row: rms of the difference (mean taken off) over the rms of the reference row; the largest."""
+    return float(row_errors(got, want).max())
+
+
+def rows_agree(got, want, dtype):
+    """32-bit: every row within the tolerance. bf16: a router's near-tie may pick another expert for a token (and what
+    reads that token shifts with it): the median row must be inside the tolerance and four rows of five within 2.5
+    times it (a wrong kernel is off by the rows' own size; the kernels are held to the sharp bound by the mechanism
+    tests)."""
+    e = row_errors(got, want)
+    if dtype in ("float32", torch.float32):
+        return bool(e.max() < tol(dtype))
+    return bool(e.median() < tol(dtype) and (e < 2.5 * tol(dtype)).double().mean() >= 0.8)
+
+
+def i32(x, device):
+    return torch.tensor(x, dtype=torch.int32, device=device)
+
+
+# ------------------------------------------------------------------------------------ mechanisms
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+def test_embedding_norm_and_closing_sum(device, dtype):
+    g = torch.Generator().manual_seed(3)
+    for T, W in ((5, 48), (3, 257), (1, 8), (2, 1030), (1, 4100)):
+        E = torch.randn(19, W, generator=g).to(dtype)
+        toks = torch.randint(0, 19, (T,), generator=g)
+        x = pb.embed_scaled(toks.to(device), E.to(device), 7.5)
+        assert x.dtype == torch.float32 and rel_err(x.cpu(), E.to(F64)[toks] * 7.5) < 1e-6
+        x = (torch.randn(T, W, generator=g) * 3 + 0.5)
+        w = (1 + 0.2 * torch.randn(W, generator=g)).to(dtype)
+        xd = x.clone().to(device)
+        x1, h32, hc = pb.sum_norm(xd, None, None, w.to(device), 1e-5, dtype, want32=True)
+        want = O.rms(x.to(F64), 1e-5) * w.to(F64)
+        assert x1 is xd and torch.equal(x1.cpu(), x) and h32.dtype == torch.float32 and hc.dtype == dtype
+        assert rel_err(h32.cpu(), want) < 1e-5 and rel_err(hc.float().cpu(), want) < tol(dtype)
+        y1, y2 = (2 * torch.randn(T, W, generator=g)).to(dtype), (2 * torch.randn(T, W, generator=g)).to(dtype)
+        for ys in ((y1, y2), (y1, None)):
+            xd = x.clone().to(device)
+            x_want = x.to(F64) + ys[0].to(F64) + (ys[1].to(F64) if ys[1] is not None else 0)
+            x2, h2, hc2 = pb.sum_norm(xd, ys[0].to(device), ys[1].to(device) if ys[1] is not None else None,
+                                      w.to(device), 1e-5, dtype, want32=True)
+            assert x2 is xd and rel_err(x2.cpu(), x_want) < 1e-6
+            assert rel_err(h2.cpu(), O.rms(x_want, 1e-5) * w.to(F64)) < 1e-5
+            assert rel_err(hc2.float().cpu(), O.rms(x_want, 1e-5) * w.to(F64)) < tol(dtype)
+        xd = x.clone().to(device)  # the last layer: the sum alone
+        x3, h3, hc3 = pb.sum_norm(xd, y1.to(device), y2.to(device), None, 1e-5, dtype)
+        assert h3 is None and hc3 is None and rel_err(x3.cpu(), x.to(F64) + y1.to(F64) + y2.to(F64)) < 1e-6
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+def test_activations_on_column_ranges(device, dtype):
+    g = torch.Generator().manual_seed(4)
+    for n, Fh, lead in ((7, 24, 5), (1, 3, 0), (33, 130, 16)):
+        wide = (2 * torch.randn(n, lead + 2 * Fh + 3, generator=g)).to(dtype)
+        gu = wide.to(device)[:, lead:lead + 2 * Fh]
+        a, b = wide[:, lead:lead + Fh].to(F64), wide[:, lead + Fh:lead + 2 * Fh].to(F64)
+        out = pb.glu_rows(gu)
+        assert out.is_contiguous() and rel_err(out.float().cpu(), torch.nn.functional.silu(a) * b) < tol(dtype)
+        z = wide.to(device)[:, lead:lead + Fh]
+        assert rel_err(pb.relu2_rows(z).float().cpu(), torch.relu(a) ** 2) < tol(dtype)
+
+
+ROTS = [{"base": 10000.0, "dims": 8}, {"base": 100.0, "dims": 16, "scaling": {"factor": 8.0, "original": 64, "fast": 16.0, "slow": 2.0}},
+        {"base": 50000.0, "dims": 6, "scaling": {"factor": 2.5, "original": 300, "fast": 32.0, "slow": 1.0}},
+        {"base": 7.0, "dims": 2, "scaling": {"factor": 1.0, "original": 10, "fast": 4.0, "slow": 1.0}}]
+
+
+@pytest.mark.parametrize("rot", ROTS)
+def test_rotation_table(rot):
+    f, m = O.rotation_frequencies(rot)
+    if rot.get("scaling") and rot["scaling"]["factor"] > 1:
+        plain, _ = O.rotation_frequencies({"base": rot["base"], "dims": rot["dims"]})
+        assert m > 1 and not torch.equal(f, plain)  # the case is no trivial one
+    tab = wattn.rotation_table(rot["base"], rot["dims"], 700, "cpu", rot.get("scaling"))
+    pos = torch.arange(700, dtype=F64).unsqueeze(1)
+    want = torch.cat([torch.cos(pos * f), torch.sin(pos * f)], 1) * m
+    assert tab.shape == (700, rot["dims"]) and float((tab.to(F64) - want).abs().max()) < 2e-7 * m
+
+
+def _paged(n_pages, G, D, V, dtype, device, fill=9.0):
+    kc, vc = wattn.alloc_window_cache(n_pages, G, D, V, dtype, device)
+    kc.fill_(fill)  # what an earlier request left behind
+    vc.fill_(-fill)
+    return kc, vc
+
+
+def _slots(pages, lo, hi, device):
+    return torch.tensor([pages[p // PAGE] * PAGE + p % PAGE for p in range(lo, hi)], dtype=torch.int64, device=device)
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+@pytest.mark.parametrize("H,G,D,V,rot", [(4, 2, 16, 8, ROTS[0]), (3, 3, 10, 5, ROTS[2]), (2, 1, 16, 16, ROTS[1]),
+                                         (1, 1, 4, 4, None), (8, 2, 64, 32, ROTS[1])])
+def test_rotation_unit_norm_value_mixing_and_cache_write(device, dtype, H, G, D, V, rot):
+    g = torch.Generator().manual_seed(H * 100 + D)
+    T, eps, pos0 = 45, 1e-4, 90
+    proj = (torch.randn(T, (H + G) * D + G * V + 7, generator=g) * 2).to(dtype)
+    vf_wide = torch.randn(T, G * V + 3, generator=g).to(dtype)
+    lam = torch.tensor([0.3], dtype=dtype)
+    pages = [5, 2, 7, 1, 6]
+    slots = _slots(pages, pos0, pos0 + T, device)
+    slots[7] = -1  # a token that caches nothing
+    table = wattn.rotation_table(rot["base"], rot["dims"], 256, device, rot.get("scaling")) if rot else None
+    p64 = proj.to(F64)
+    for mixing in (False, True):
+        kc, vc = _paged(9, G, D, V, dtype, device)
+        vf = vf_wide.to(device)[:, 2:2 + G * V] if mixing else None
+        q = wattn.rot_norm_cache_write(proj.to(device), i32(list(range(pos0, pos0 + T)), device), table, slots, kc, vc,
+                                       H, eps, vf, lam.to(device) if mixing else None)
+        for t in range(T):
+            qh, kh = p64[t, :H * D].view(H, D), p64[t, H * D:(H + G) * D].view(G, D)
+            if rot:
+                qh, kh = O.rotate(qh, pos0 + t, rot), O.rotate(kh, pos0 + t, rot)
+            assert rel_err(q[t].float().cpu(), O.rms(qh, eps)) < tol(dtype)
+            v = p64[t, (H + G) * D:(H + G) * D + G * V]
+            if mixing:
+                v = (1 - float(lam.to(F64))) * v + float(lam.to(F64)) * vf_wide.to(F64)[t, 2:2 + G * V]
+            s = int(slots[t])
+            if s < 0:
+                continue
+            assert rel_err(kc[s // PAGE, :, s % PAGE].float().cpu(), O.rms(kh, eps)) < tol(dtype)
+            assert rel_err(vc[s // PAGE, :, s % PAGE].float().cpu().reshape(1, -1), v.reshape(1, -1)) < tol(dtype)
+        untouched = [p for p in range(9) if p not in pages]
+        assert bool((kc[untouched] == 9.0).all()) and bool((vc[untouched] == -9.0).all())
+
+
+def _attention_case(H, G, D, V, window, keep, scale, n, probes, seed, rot=None):
+    """Queries, keys and values of one sequence as the columns of an identity-like projection, so that the oracle's
+    mixer and the ops see the same numbers. `probes`: (query position, key position) pairs whose score is made to
+    stand out: a key just outside a window then shows as a row that is off by its own size."""
+    g = torch.Generator().manual_seed(seed)
+    width = (H + G) * D + G * V
+    h = torch.randn(n, width, generator=g)
+    h[:, H * D:(H + G) * D] *= 0.3
+    for qi, kj in probes:
+        for c in range(G):
+            h[kj, H * D + c * D:H * D + (c + 1) * D] = 3.0 * h[qi, c * (H // G) * D:c * (H // G) * D + D]
+    eye = torch.eye(width, dtype=F64)
+    w = {"q": eye[:H * D], "k": eye[H * D:(H + G) * D], "v": eye[(H + G) * D:], "o": torch.eye(H * V, dtype=F64)}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": scale, "mask": {"size": window, "keep_first": keep}}
+    if rot:
+        m["rot"] = rot
+    return h, w, m
+
+
+def _run_attention(h, m, dtype, device, portions, pages, nsplit=1, matrix_cores=True):
+    """The ops over a paged cache, the sequence fed in portions; returns [n, H V]."""
+    H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    rot = m.get("rot")
+    n = h.shape[0]
+    kc, vc = _paged(max(pages) + 2, G, D, V, dtype, device, fill=50.0)
+    table = wattn.rotation_table(rot["base"], rot["dims"], n + 1, device, rot.get("scaling")) if rot else None
+    shape = wattn.ScoreShape(scale=m["scale"], window=m["mask"]["size"], keep_first=m["mask"]["keep_first"])
+    bt = torch.tensor([pages], dtype=torch.int32, device=device)
+    outs, at = [], 0
+    hd = h.to(dtype).to(device)
+    for c in portions:
+        c = min(c, n - at)
+        if c <= 0:
+            break
+        q = wattn.rot_norm_cache_write(hd[at:at + c], i32(list(range(at, at + c)), device), table,
+                                       _slots(pages, at, at + c, device), kc, vc, H, 1e-6)
+        o = wattn.window_attention(q, kc, vc, bt, i32([0, c], device), i32([at + c], device), c, shape, None,
+                                   nsplit=nsplit if c == 1 else 1, matrix_cores=matrix_cores)
+        outs.append(o.reshape(c, H * V).float().cpu())
+        at += c
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+@pytest.mark.parametrize("H,G,D,V,window,keep", [(4, 2, 16, 8, 37, 3), (2, 1, 8, 8, 32, 1), (3, 3, 12, 20, 5, 40),
+                                                 (1, 1, 16, 4, 64, 0), (2, 2, 8, 8, 1, 2), (4, 1, 64, 32, 33, 6),
+                                                 (2, 1, 64, 64, 70, 33), (2, 2, 16, 16, 0, 0)])
+def test_window_keeps_first_tokens_edges_pages_portions_and_splits(device, dtype, H, G, D, V, window, keep):
+    n = 150
+    w_eff = window if window > 0 else n
+    probes = []
+    for qi in (n - 1, n - 2, 100, 97, 64, 63, 33, 32, 31):
+        probes += [(qi, qi - w_eff + 1), (qi, qi - w_eff)]  # the window's last key, and the first one outside it
+        probes += [(qi, keep - 1), (qi, keep)]  # the last kept token, and the first one that is not kept
+        probes += [(qi, 1), (qi, qi - 31), (qi, qi - 32), (qi, qi - 33)]  # far back; around a page's border
+    probes = [(a, b) for a, b in probes if 0 <= b <= a]
+    for k, (qi, kj) in enumerate(probes):
+        h, w, m = _attention_case(H, G, D, V, window, keep, 4.0 / math.sqrt(D) * 3, n, [(qi, kj)], 7 + k % 3)
+        if dtype == torch.bfloat16:  # the oracle sees what the kernels see
+            h = h.to(dtype).float()
+        want, _ = O.attention_mixer(h.to(F64)[:qi + 1], w, m, 1e-6, None)
+        pages = [3, 1, 4, 9, 2][:(n + PAGE - 1) // PAGE]
+        for portions, nsplit in (([n], 1), ([qi, 1, n], 1), ([qi, 1, n], 3), ([max(qi - 1, 1), 2, n], 1)):
+            if k % 4 != len(portions) % 4 and portions != [qi, 1, n]:
+                continue  # every probe as a decoded token; the other ways of cutting in turn
+            got = _run_attention(h, m, dtype, device, portions, pages, nsplit)
+            assert rel_err(got[qi:qi + 1], want[qi:qi + 1]) < tol(dtype), (qi, kj, portions, nsplit)
+    # a whole sequence with rotation, cut in several ways, on both kernels for prompt portions
+    h, w, m = _attention_case(H, G, D, V, window, keep, 1.0 / math.sqrt(D), n, [], 1,
+                              rot={"base": 100.0, "dims": min(D, 8), "scaling": {"factor": 4.0, "original": 32,
+                                                                                  "fast": 8.0, "slow": 1.0}})
+    if dtype == torch.bfloat16:
+        h = h.to(dtype).float()
+    want, _ = O.attention_mixer(h.to(F64), w, m, 1e-6, None)
+    for portions, mc in (([n], True), ([n], False), ([1], True), ([2], True), ([3, 17, 1, 1, 64, 31, 2, 33], True),
+                         ([70, 1], True)):
+        got = _run_attention(h, m, dtype, device, portions + [portions[-1]] * n, [6, 0, 3, 8, 1], 2, mc)
+        assert rel_err(got, want) < tol(dtype), (portions, mc)
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+@pytest.mark.parametrize("H,D,V,decay", [(3, 16, 24, [0.5, 0.97, 1.0]), (1, 8, 8, [0.999]), (2, 40, 70, [0.0, 0.9]),
+                                         (2, 64, 64, [0.8, 0.99]), (1, 128, 32, [0.95]), (1, 130, 16, [0.9])])
+def test_lightning_portions_rows_and_slots_used_again(device, dtype, H, D, V, decay):
+    g = torch.Generator().manual_seed(D)
+    n, n_slots, lead = 150, 4, 3
+    N = 2 * H * D + 2 * H * V
+    wide = torch.randn(n, lead + N + 2, generator=g).to(dtype)
+    proj = wide[:, lead:lead + N]
+    wn = (1 + 0.2 * torch.randn(H * V, generator=g)).to(dtype)
+    eye = torch.eye(N, dtype=F64)
+    a, b, c = H * D, 2 * H * D, 2 * H * D + H * V
+    w = {"q": eye[:a], "k": eye[a:b], "v": eye[b:c], "g": eye[c:], "norm": wn.to(F64), "o": torch.eye(H * V, dtype=F64)}
+    m = {"heads": H, "dim": D, "vdim": V, "decay": decay}
+    want, S_want = O.lightning_mixer(proj.to(F64), w, m, 1e-5)
+    state = lightning_ops.alloc_state(n_slots, H, D, V, device)
+    state.fill_(1e3)  # what an earlier request left
+    lam = torch.tensor(decay, dtype=torch.float32, device=device)
+    pd = wide.to(device)[:, lead:lead + N]
+
+    def run(portions, slot):
+        outs, at = [], 0
+        for cnt in portions:
+            cnt = min(cnt, n - at)
+            if cnt <= 0:
+                break
+            rows = pd[at:at + cnt]
+            o = lightning_ops.lightning_scan(rows, 0, a, b, lam, i32([0, cnt], device), i32([at], device),
+                                             i32([slot], device), state, max_q=cnt)
+            outs.append(lightning_ops.lightning_out(o, rows[:, c:], wn.to(device), 1e-5).float().cpu())
+            at += cnt
+        return torch.cat(outs)
+
+    for k, sizes in enumerate(([n], [1] * n, [2] * n, [3, 1, 17, 2, 1, 64, 16, 40, 6], [100, 1] + [1] * n,
+                               [64, 64, 22], [16] * n)):
+        got = run(sizes, k % n_slots)
+        assert rel_err(got, want) < tol(dtype), sizes[:4]
+        assert rel_err(state[k % n_slots].reshape(1, -1).cpu(), S_want.reshape(1, -1)) < 1e-4
+    # two sequences side by side at different places, beside a row that owns no slot
+    state.fill_(-7.0)
+    first = run([20], 0)
+    before = state.clone()
+    both = torch.cat([pd[20:23], pd[:40], pd[:2]]).contiguous()
+    o = lightning_ops.lightning_scan(both, 0, a, b, lam, i32([0, 3, 43, 45], device), i32([20, 0, 0], device),
+                                     i32([0, 3, -1], device), state, max_q=40)
+    out = lightning_ops.lightning_out(o, both[:, c:], wn.to(device), 1e-5).float().cpu()
+    assert bool((o[43:] == 0).all())
+    assert rel_err(torch.cat([first, out[:3]]), want[:23]) < tol(dtype) and rel_err(out[3:43], want[:40]) < tol(dtype)
+    assert torch.equal(state[[1, 2]], before[[1, 2]])
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+@pytest.mark.parametrize("W,ff,E,top,shared", [(48, 20, 5, 2, 12), (24, 8, 3, 3, 0), (64, 64, 4, 1, 64), (50, 9, 7, 3, 5),
+                                               (32, 16, 1, 1, 8)])
+def test_routed_and_shared_experts(device, dtype, W, ff, E, top, shared):
+    g = torch.Generator().manual_seed(W + E)
+    mod = RoutedSwiGLUExperts(W, ff, E, top, shared, dtype, device)
+    with torch.no_grad():
+        for p in mod.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) / (p.shape[-1] ** 0.5 if p.dim() > 1 else 1.0)).to(dtype))
+        mod.router.mul_(4.0)  # clear choices: a near-tie would let bf16 pick another expert than the oracle
+    w = {"router": mod.router, "router.b": mod.router_bias}
+    for i in range(E):
+        w[f"e{i}.gate"], w[f"e{i}.up"], w[f"e{i}.down"] = mod.gate_up[i, :ff], mod.gate_up[i, ff:], mod.down[i]
+    e = {"router": {"experts": E, "top": top}, "expert": {"ff": ff}}
+    sh_in = torch.randn(2 * shared, W, generator=g).to(dtype) / W ** 0.5
+    if shared:
+        e["shared"] = {"ff": shared}
+        w["shared.gate"], w["shared.up"], w["shared.down"] = sh_in[:shared], sh_in[shared:], mod.shared_down
+    w = {k: v.detach().to(F64).cpu() for k, v in w.items()}
+    for T in (1, 9, 70):
+        h = torch.randn(T, W, generator=g).to(dtype)
+        want = O.moe_ff(h.to(F64), w, e)
+        hd = h.to(device)
+        cols = torch.nn.functional.linear(hd, sh_in.to(device))
+        with torch.no_grad():
+            got = mod(cols, hd, hd.float())
+        assert rows_agree(got.float().cpu(), want, dtype), rel_err(got.float().cpu(), want)
+
+
+# ------------------------------------------------------------------------------------ whole models through the engine
+def attn(heads=4, kv=2, dim=16, vdim=8, window=37, keep=3, rot_dims=8, scale=0.4, v_mix=True, base=10000.0, factor=4.0,
+         original=64, mlp="moe", ff=24, experts=5, top=2, shared=12):
+    mixer = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale, "v_mix": v_mix,
+             "mask": {"size": window, "keep_first": keep}}
+    if rot_dims:
+        mixer["rot"] = {"base": base, "dims": rot_dims}
+        if factor:
+            mixer["rot"]["scaling"] = {"factor": factor, "original": original, "fast": 16.0, "slow": 1.0}
+    return {"type": "attention", "mixer": mixer, "mlp": ffn(mlp, ff, experts, top, shared)}
+
+
+def light(heads=3, dim=16, vdim=24, decay=(0.6, 0.95, 0.999), mlp="dense", ff=40, experts=5, top=2, shared=12):
+    return {"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": list(decay)},
+            "mlp": ffn(mlp, ff, experts, top, shared)}
+
+
+def ffn(kind, ff, experts, top, shared):
+    if kind is None:
+        return None
+    if kind == "dense":
+        return {"kind": "dense", "ff": ff}
+    d = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if shared:
+        d["shared"] = {"ff": shared}
+    return d
+
+
+def config(layers, width=48, vocab=101, eps=1e-5, scale=6.0):
+    return {"architecture": "Pobelorn", "embedding": {"scale": scale}, "layers": layers, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}
+
+
+MIXED = config([attn(mlp="dense", ff=40), light(mlp="moe"), attn(window=5, keep=0), attn(heads=2, kv=2, v_mix=False, mlp=None),
+                light(heads=2, dim=8, vdim=8, decay=(0.9, 1.0), mlp=None), attn(window=64, keep=9, experts=3, top=3, shared=0)])
+
+
+def make_engine(cfg_dict, device, dtype, num_pages=40, max_running=4, context=512, score=True, graphs=True):
+    cfg = ModelConfig.from_hf_dict(cfg_dict)
+    srv = InferenceServerConfig(model_path="", dtype=dtype, context_length=context, max_running_requests=max_running,
+                                num_continuous_decode_steps=1, max_prefill_tokens=context,
+                                disable_cuda_graph=not graphs)
+    eng = NativeInferenceEngine(srv, model_config=cfg, device=torch.device(device), num_pages=num_pages,
+                                score_mode=score)
+    eng.initialize(load_weights=False)
+    weights = {k: v.detach().float().cpu() for k, v in eng.model.checkpoint_tensors().items()}
+    return eng, weights
+
+
+def replay(eng, steps):
+    """steps: list of lists of (request id, tokens, wanted places, ends after this step) -> {id: {position: logits}}."""
+    out, fed, live = {}, {}, set()
+    for step in steps:
+        for rid, toks, want, _ in step:
+            if rid not in live:
+                eng.open_replay(rid)
+                live.add(rid)
+                fed[rid] = 0
+        logits = eng.replay_step([(rid, toks, want) for rid, toks, want, _ in step])
+        at = 0
+        for rid, toks, want, end in step:
+            for w in want:
+                out.setdefault(rid, {})[fed[rid] + w] = logits[at]
+                at += 1
+            fed[rid] += len(toks)
+            if end:
+                eng.close_replay(rid)
+                live.discard(rid)
+        assert at == logits.shape[0]
+    return out
+
+
+def cut(rid, tokens, sizes):
+    """One request alone, fed in portions of the given sizes (the last size repeats); every position is wanted."""
+    steps, at, i = [], 0, 0
+    while at < len(tokens):
+        c = min(sizes[min(i, len(sizes) - 1)], len(tokens) - at)
+        steps.append([(rid, tokens[at:at + c], list(range(c)), at + c == len(tokens))])
+        at += c
+        i += 1
+    return steps
+
+
+def check_against_oracle(got, tokens, weights, cfg_dict, dtype, rid):
+    want, _ = O.forward(cfg_dict, weights, tokens)
+    rows = torch.from_numpy(np.stack([got[rid][p] for p in range(len(tokens))]))
+    assert rows_agree(rows, want, dtype), rel_err(rows, want)
+
+
+def tokens_of(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_whole_prompt_and_every_layer(device, dtype):
+    eng, w = make_engine(MIXED, device, dtype)
+    try:
+        toks = tokens_of(75, MIXED["vocab"], 1)
+        eng.runner.layer_trace = []
+        got = replay(eng, cut("a", toks, [len(toks)]))
+        trace, eng.runner.layer_trace = eng.runner.layer_trace, None
+        _, layers = O.forward(MIXED, w, toks)
+        assert len(trace) == len(layers) == 6
+        for a, b in zip(trace, layers):
+            assert rows_agree(a.cpu(), b, dtype)
+        check_against_oracle(got, toks, w, MIXED, dtype, "a")
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_prefill_against_token_by_token_and_portions(device, dtype):
+    eng, w = make_engine(MIXED, device, dtype)
+    try:
+        toks = tokens_of(140, MIXED["vocab"], 2)
+        for k, sizes in enumerate(([1], [60, 1], [2], [3, 64, 2, 31, 33, 1, 1, 5], [1, 32, 32, 32, 1], [17, 16])):
+            got = replay(eng, cut(f"r{k}", toks, list(sizes)))
+            check_against_oracle(got, toks, w, MIXED, dtype, f"r{k}")
+        assert eng.sched.num_free_state_slots() == 4 and eng.sched.num_free_pages() == eng.sched.num_total_pages()
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_unequal_requests_in_one_batch_with_pages_and_slots_used_again(device, dtype):
+    """Seven requests of very different lengths through three slots and a pool that cannot hold them all at once:
+    portions of some beside single tokens of others; each must equal the request computed alone."""
+    eng, w = make_engine(MIXED, device, dtype, num_pages=15, max_running=3)
+    try:
+        V = MIXED["vocab"]
+        reqs = {f"q{i}": tokens_of(n, V, 10 + i) for i, n in enumerate((1, 70, 23, 130, 2, 97, 40))}
+        plan = {"q0": [1], "q1": [5, 1, 1, 33, 2, 1], "q2": [23], "q3": [64, 2, 1, 1, 40, 1], "q4": [1, 1], "q5": [31, 33, 1],
+                "q6": [2, 1]}
+        waiting, live, at, steps = list(reqs), [], {r: 0 for r in reqs}, []
+        nth = {r: 0 for r in reqs}
+        while waiting or live:
+            while waiting and len(live) < 3:
+                need = sum((len(reqs[r]) + 31) // 32 for r in live) + (len(reqs[waiting[0]]) + 31) // 32
+                if need > 13:
+                    break
+                live.append(waiting.pop(0))
+            step = []
+            for r in list(live):
+                sizes = plan[r]
+                c = min(sizes[min(nth[r], len(sizes) - 1)], len(reqs[r]) - at[r])
+                end = at[r] + c == len(reqs[r])
+                step.append((r, reqs[r][at[r]:at[r] + c], list(range(c)), end))
+                at[r] += c
+                nth[r] += 1
+                if end:
+                    live.remove(r)
+            steps.append(step)
+        assert max(len(s) for s in steps) == 3 and any(len(t) == 1 for s in steps if len(s) > 1 for _, t, _, _ in s)
+        got = replay(eng, steps)
+        for r, toks in reqs.items():
+            check_against_oracle(got, toks, w, MIXED, dtype, r)
+        assert eng.sched.num_free_state_slots() == 3 and eng.sched.num_free_pages() == eng.sched.num_total_pages()
+    finally:
+        eng.destroy()
+
+
+SHAPES = [
+    # one head everywhere, key size = value size = rotated size = width of the expert, as many experts as are chosen,
+    # an embedding factor and a decay of 1: values that hide mix-ups
+    config([attn(1, 1, 16, 16, 33, 1, 16, mlp="moe", ff=16, experts=2, top=2, shared=16), light(1, 16, 16, (1.0,), ff=16)],
+           width=16, scale=1.0),
+    # sizes that are no multiples of 8 or of each other, a window of one token and one beyond the sequence, no
+    # rotation in one layer and no stretching in another, more kept tokens than the window is wide
+    config([light(5, 12, 20, (0.3, 0.5, 0.7, 0.9, 0.99), mlp="moe", ff=10, experts=3, top=1, shared=7),
+            attn(6, 3, 12, 20, 1, 11, 6, scale=0.11, base=500.0, factor=0, mlp="dense", ff=30),
+            attn(6, 3, 10, 20, 500, 0, 0, scale=0.9, mlp=None),
+            attn(3, 1, 20, 60, 7, 2, 20, v_mix=False, factor=16.0, original=16, experts=7, top=3, shared=0)],
+           width=40, vocab=67, eps=1e-3, scale=0.5),
+    config([attn(4, 4, 16, 24, 0, 0)], width=24),  # every earlier token seen
+    config([light(2, 8, 8, (0.5, 0.75), mlp=None), light(4, 32, 16, (0.9, 0.9, 0.99, 0.2), mlp="moe")], width=56),
+    # nothing a multiple of 4: width, head sizes, expert widths, vocabulary
+    config([attn(3, 1, 10, 14, 13, 5, 6, ff=9, experts=4, top=2, shared=5), light(7, 6, 5, [0.9] * 7, mlp="dense", ff=11),
+            attn(3, 1, 6, 14, 3, 1, 2, mlp=None)], width=50, vocab=59),
+    # sizes the matrix-core paths take
+    config([attn(4, 2, 64, 64, 40, 4, 32, ff=64, experts=4, top=2, shared=64), light(2, 64, 64, (0.9, 0.99), ff=128),
+            attn(8, 2, 128, 32, 70, 33, 64, v_mix=False, mlp="dense", ff=128), light(1, 128, 128, (0.97,), mlp=None),
+            attn(4, 2, 128, 64, 50, 0, 128, mlp=None)], width=64),
+]
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("which", range(len(SHAPES)))
+def test_other_sizes_windows_constants_and_orders(device, dtype, which):
+    cfg = SHAPES[which]
+    eng, w = make_engine(cfg, device, dtype)
+    try:
+        toks = tokens_of(90, cfg["vocab"], 20 + which)
+        check_against_oracle(replay(eng, cut("w", toks, [len(toks)])), toks, w, cfg, dtype, "w")
+        check_against_oracle(replay(eng, cut("c", toks, [7, 2, 33, 1, 1, 20, 1])), toks, w, cfg, dtype, "c")
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_first_tokens_and_long_decoding(device, dtype):
+    cfg = config([attn(window=40, keep=2), light(), attn(heads=2, kv=2, window=9, keep=4, mlp=None)])
+    eng, w = make_engine(cfg, device, dtype)
+    try:
+        for n in (1, 2, 3, 5):
+            toks = tokens_of(n, cfg["vocab"], 40 + n)
+            check_against_oracle(replay(eng, cut(f"s{n}", toks, [1])), toks, w, cfg, dtype, f"s{n}")
+            check_against_oracle(replay(eng, cut(f"w{n}", toks, [n])), toks, w, cfg, dtype, f"w{n}")
+        toks = tokens_of(230, cfg["vocab"], 44)  # the windows pass over decoded tokens several times
+        check_against_oracle(replay(eng, cut("long", toks, [20, 1])), toks, w, cfg, dtype, "long")
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_greedy_generation_through_the_engine(device, dtype):
+    """The engine's own entry point: prompts of unequal length generated together, prefill plans, then decode
+    plans (captured graphs on the GPU), more requests than request slots."""
+    cfg = config([attn(window=21, keep=2), light(mlp="moe"), attn(heads=2, kv=1, dim=16, vdim=16, window=70, v_mix=False,
+                                                                            mlp=None)], vocab=61)
+    eng, w = make_engine(cfg, device, dtype, max_running=3, score=False)
+    try:
+        prompts = [tokens_of(n, cfg["vocab"], 50 + n) for n in (3, 41, 18, 1, 66)]
+        res = eng.generate_blocking(prompts, max_new_tokens=12, greedy=True)
+        agree = 0
+        for p, r in zip(prompts, res):
+            assert r.finish_reason == "length" and len(r.output_tokens) == 12
+            want = O.greedy(cfg, w, p, 12)
+            if dtype == "float32":
+                assert r.output_tokens == want
+            else:  # a near-tie (of two tokens, of two experts) may flip under bf16
+                agree += r.output_tokens[0] == want[0]
+        assert dtype == "float32" or agree >= 4
+        assert eng.sched.num_free_state_slots() == 3
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_served_from_a_checkpoint_directory(device, tmp_path):
+    """The framework's own path from a directory with config.json and model.safetensors: the model class is chosen by
+    the configuration, the weights come through the engine's loader; several decode steps per plan."""
+    from areal_vllm_amd.models import build_model
+
+    cfg_dict = config([attn(2, 1, 8, 16, 9, 2, 4, ff=12, experts=3, top=2, shared=6), light(2, 8, 8, (0.8, 0.99), ff=20)],
+                      width=32, vocab=53)
+    m = build_model(ModelConfig.from_hf_dict(cfg_dict), dtype=torch.bfloat16)
+    m.flatten()
+    m.init_weights(seed=9)
+    m.save_checkpoint(str(tmp_path))
+    w = {k: v.float() for k, v in m.checkpoint_tensors().items()}
+    srv = InferenceServerConfig(model_path=str(tmp_path), dtype="float32", context_length=128, max_running_requests=2,
+                                num_continuous_decode_steps=2)
+    eng = NativeInferenceEngine(srv, device=torch.device(device), num_pages=12)
+    eng.initialize()
+    try:
+        prompts = [tokens_of(n, 53, 70 + n) for n in (5, 33, 17)]
+        res = eng.generate_blocking(prompts, max_new_tokens=7, greedy=True)
+        for p, r in zip(prompts, res):
+            assert r.output_tokens == O.greedy(cfg_dict, w, p, 7)
+    finally:
+        eng.destroy()
+
+
+def test_config_reader_and_checkpoint_save_then_load(tmp_path):
+    cfg = ModelConfig.from_hf_dict(SHAPES[1])
+    assert cfg.family == "pobelorn" and cfg.n_layers == 4 and cfg.has_recurrent_state and cfg.tie_word_embeddings
+    assert not ModelConfig.from_hf_dict(SHAPES[2]).has_recurrent_state
+    from areal_vllm_amd.models import build_model
+
+    m = build_model(cfg, dtype=torch.float32)
+    m.flatten()
+    m.init_weights(seed=4)
+    # every attention layer carries its mixing number; the ones that never read it are not counted
+    unused = sum(1 for b in m.layers if b.kind == "attention" and b.mix.v_mix != "mix")
+    assert sum(p.numel() for p in m.parameters()) == cfg.n_params() + unused
+    assert [b.mix.v_mix for b in m.layers if b.kind == "attention"] == ["first", "mix", None]
+    m.save_checkpoint(str(tmp_path))
+    cfg2 = ModelConfig.from_pretrained(str(tmp_path))
+    assert cfg2.layers == cfg.layers and cfg2.embed_scale == cfg.embed_scale == 0.5
+    m2 = build_model(cfg2, dtype=torch.float32)
+    m2.flatten()
+    m2.load_checkpoint(str(tmp_path))
+    for (n1, a), (n2, b) in zip(m.checkpoint_tensors().items(), m2.checkpoint_tensors().items()):
+        assert n1 == n2 and torch.equal(a, b)
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf_dict(config([dict(attn(), type="conv")]))
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf_dict(config([light(heads=2, decay=(0.5,))]))
