@@ -9,6 +9,10 @@ plans and generated tokens/s over the decode plans (the engine's own clocks), an
 The Lufivik design (latent attention with a sliding window, routed clamped-GLU experts, sublayers between two layer
 norms) is compared the same way with a Qwen3-MoE-style transformer: the same width, depth, heads, experts and experts
 per token, its experts as wide as the parameter budget allows.
+
+The Pobelorn design (parallel blocks; window attention on rotated unit-norm queries and keys that keeps the first
+tokens, every third layer lightning attention; routed + shared gated experts, the first layer a squared-ReLU MLP) is
+compared with the same kind of twin.
 """
 import json
 import sys
@@ -29,6 +33,13 @@ LUFIVIK_SIZES = {
     "w1024": (1024, 4, 8, 64, 32, 64, 384, 256, 512, 16, 2, 512),
     "w2048": (2048, 4, 16, 128, 64, 128, 768, 512, 1024, 32, 4, 768),
     "w4096": (4096, 2, 32, 128, 64, 128, 1536, 512, 1024, 64, 4, 1024),
+}
+# Pobelorn: width, layers, heads, kv heads, head size (keys, values), rotated coordinates, window, kept first tokens,
+# experts, experts per token, expert width, shared expert width
+POBELORN_SIZES = {
+    "w1024": (1024, 4, 8, 2, 128, 64, 512, 4, 16, 2, 512, 512),
+    "w2048": (2048, 4, 16, 4, 128, 64, 1024, 4, 32, 4, 768, 768),
+    "w4096": (4096, 2, 32, 8, 128, 64, 1024, 4, 64, 4, 1024, 1024),
 }
 VOCAB = 32768
 
@@ -56,6 +67,25 @@ def lufivik_dict(width, layers, heads, dim, rot, vdim, q_rank, kv_rank, window, 
     return {"architecture": "Lufivik", "layers": [json.loads(json.dumps(layer)) for _ in range(layers)],
             "norm": {"eps": 1e-5}, "canon": {"taps": 4},
             "embedding": {"bigram": {"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}}, "vocab": VOCAB, "width": width}
+
+
+def pobelorn_dict(width, layers, heads, kv, dim, rot, window, keep, experts, top, ff, shared) -> Dict[str, Any]:
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": shared}}
+    ls = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": 4 * width} if i == 0 and layers > 2 else json.loads(json.dumps(moe))
+        if i % 3 == 1:
+            ls.append({"type": "lightning", "mlp": mlp,
+                       "mixer": {"heads": heads, "dim": dim, "vdim": dim,
+                                 "decay": [1.0 - 2.0 ** (-(3.0 + 6.0 * (h + 1) / heads)) for h in range(heads)]}})
+        else:
+            ls.append({"type": "attention", "mlp": mlp,
+                       "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                 "v_mix": True, "mask": {"size": window, "keep_first": keep},
+                                 "rot": {"base": 10000.0, "dims": rot,
+                                         "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}})
+    return {"architecture": "Pobelorn", "embedding": {"scale": float(width) ** 0.5}, "layers": ls, "norm": {"eps": 1e-6},
+            "vocab": VOCAB, "width": width}
 
 
 def moe_twin_config(lcfg, width, layers, heads, experts, top):
@@ -117,6 +147,26 @@ def measure(cfg, n_prompts: int, prompt_len: int, new_tokens: int, device) -> Di
     return out
 
 
+def run_pobelorn(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, dev) -> int:
+    from ..models.config import ModelConfig
+
+    for name in sizes:
+        width, layers, heads, kv, dim, rot, window, keep, experts, top, ff, shared = POBELORN_SIZES[name]
+        pcfg = ModelConfig.from_hf_dict(pobelorn_dict(*POBELORN_SIZES[name]))
+        tcfg = moe_twin_config(pcfg, width, layers, heads, experts, top)
+        row = {"design": "pobelorn", "size": name, "width": width, "layers": layers, "heads": heads, "kv_heads": kv,
+               "head_dim": dim, "rot_dims": rot, "window": window, "keep_first": keep, "experts": experts, "top": top,
+               "expert_ff": ff, "shared_ff": shared, "twin_expert_ff": tcfg.moe_intermediate_size, "prompts": n_prompts,
+               "prompt_len": prompt_len, "new_tokens": new_tokens, "dtype": "bf16", "data": "synthetic"}
+        for label, cfg in (("pobelorn", pcfg), ("qwen3_moe_twin", tcfg)):
+            m = measure(cfg, n_prompts, prompt_len, new_tokens, dev)
+            row[label] = {"params_no_embedding": cfg.n_params(with_embedding=False), **{k: round(v, 1) for k, v in m.items()}}
+        row["prefill_ratio"] = round(row["pobelorn"]["prefill_tok_s"] / row["qwen3_moe_twin"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["pobelorn"]["decode_tok_s"] / row["qwen3_moe_twin"]["decode_tok_s"], 3)
+        print(json.dumps(row), flush=True)
+    return 0
+
+
 def run_lufivik(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, dev) -> int:
     from ..models.config import ModelConfig
 
@@ -143,6 +193,8 @@ def run(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, devi
     dev = torch.device(device, 0) if device == "cuda" else torch.device(device)
     if design == "lufivik":
         return run_lufivik(sizes, n_prompts, prompt_len, new_tokens, dev)
+    if design == "pobelorn":
+        return run_pobelorn(sizes, n_prompts, prompt_len, new_tokens, dev)
     for name in sizes:
         width, layers, heads, kv, dim, ff, window = SIZES[name]
         kcfg = ModelConfig.from_hf_dict(kuzanex_dict(width, layers, heads, kv, dim, ff, window))

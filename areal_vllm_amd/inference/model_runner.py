@@ -881,7 +881,10 @@ class HybridModelRunner(ModelRunner):
                 G, D, V = blk.mix.cache_shape()
                 if hasattr(blk.mix, "prepare"):  # mixers that rotate by position
                     blk.mix.prepare(self.max_context + 1, tables, self.device)
-                self.kv.append(wattn.alloc_window_cache(self.num_pages, G, D, V, self.dtype, self.device))
+                if hasattr(blk.mix, "alloc_cache"):  # mixers that choose their page layout
+                    self.kv.append(blk.mix.alloc_cache(self.num_pages, self.dtype, self.device))
+                else:
+                    self.kv.append(wattn.alloc_window_cache(self.num_pages, G, D, V, self.dtype, self.device))
                 self.state.append(None)
             elif blk.kind == "lightning":
                 from ..ops import lightning as lightning_ops
@@ -1045,7 +1048,8 @@ class HybridModelRunner(ModelRunner):
             return nsplit, ws
         mixers = [blk.mix for blk in self.model.layers if blk.kind == "attention"]
         if mixers and self.device.type == "cuda":
-            nsplit = max(wattn.decode_splits(Bp, m.shape.window, self.max_context, m.shape.keep_first) for m in mixers)
+            nsplit = max(m.decode_splits(Bp, self.max_context) if hasattr(m, "decode_splits") else
+                         wattn.decode_splits(Bp, m.shape.window, self.max_context, m.shape.keep_first) for m in mixers)
             if nsplit > 1:
                 hv = max(m.H * m.V for m in mixers)
                 hh = max(m.H for m in mixers)

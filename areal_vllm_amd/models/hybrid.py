@@ -282,7 +282,16 @@ class StepTensors:
         self.block_tables, self.first_pos, self.state_slots = block_tables, first_pos, state_slots
         self.nsplit, self.workspace = int(nsplit), workspace
         self.positions = positions  # position of every token (int32), for mixers that rotate by position
+        self._cu_k = None
         self.v_first = None  # this step's values of the first value-sharing attention layer [T, G Dv] (set by it)
+
+
+    @property
+    def cu_k(self) -> torch.Tensor:
+        """Cumulative context lengths int32 [B + 1] (formed once per step)."""
+        if self._cu_k is None:
+            self._cu_k = F.pad(torch.cumsum(self.ctx_len, 0, dtype=torch.int32), (1, 0))
+        return self._cu_k
 
 
 class WindowAttentionMixer(nn.Module):
@@ -451,6 +460,7 @@ class RotaryWindowAttentionMixer(nn.Module):
         self.v_mix = v_mix
         self.vmix = nn.Parameter(torch.zeros(1, dtype=dtype, device=device))  # read by "mix" layers only
         self.table: Optional[torch.Tensor] = None
+        self.standard = False  # the cache is in the engine's standard layout (`alloc_cache`)
 
     def in_rows(self) -> int:
         return (self.H + self.G) * self.D + self.G * self.V
@@ -460,6 +470,25 @@ class RotaryWindowAttentionMixer(nn.Module):
 
     def cache_shape(self):
         return self.G, self.D, self.V
+
+    def alloc_cache(self, num_pages: int, dtype, device):
+        """Paged K / V of this layer: the engine's standard layout (and its flash / paged-decode kernels) for bf16
+        heads of 128 on the GPU, otherwise token-major pages of any key and value size."""
+        from ..ops.attention import alloc_kv_cache
+
+        self.standard = wattn.standard_layout_ok(self.D, self.V, dtype, device)
+        if self.standard:
+            return alloc_kv_cache(num_pages, self.G, self.D, dtype, device)
+        return wattn.alloc_window_cache(num_pages, self.G, self.D, self.V, dtype, device)
+
+    def decode_splits(self, batch: int, max_context: int) -> int:
+        if self.standard:
+            from ..ops.attention import decode_num_splits
+
+            w = self.shape.window
+            span = max_context if w <= 0 else min(w + wattn.PAGE_SIZE + self.shape.keep_first, max_context)
+            return decode_num_splits(batch, self.G, span)
+        return wattn.decode_splits(batch, self.shape.window, max_context, self.shape.keep_first)
 
     def prepare(self, n_pos: int, tables: Dict[Any, torch.Tensor], device):
         """The rotation table for positions below `n_pos`; mixers with the same constants share one."""
@@ -482,9 +511,15 @@ class RotaryWindowAttentionMixer(nn.Module):
         elif self.v_mix == "mix":
             vf, lam = st.v_first, self.vmix
             assert vf is not None and vf.shape[1] == G * V, "the value-sharing layers need equal key/value head layouts"
-        q = wattn.rot_norm_cache_write(proj, st.positions, self.table, st.slots, kc, vc, H, self.eps, vf, lam)
-        o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
-                                   nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace)
+        q = wattn.rot_norm_cache_write(proj, st.positions, self.table, st.slots, kc, vc, H, self.eps, vf, lam,
+                                       v_transposed=self.standard)
+        nsplit = st.nsplit if st.max_q == 1 else 1
+        if self.standard:
+            o = wattn.window_attention_standard(q, kc, vc, st.block_tables, st.cu_q, st.cu_k, st.ctx_len, st.max_q,
+                                                self.shape, nsplit=nsplit, workspace=st.workspace)
+        else:
+            o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
+                                       nsplit=nsplit, workspace=st.workspace)
         return o.view(proj.shape[0], H * V)
 
 

@@ -99,14 +99,16 @@ def rotation_table(base: float, dims: int, n_pos: int, device, scaling: Optional
 
 def rot_norm_cache_write(proj: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
                          slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, n_heads: int, eps: float,
-                         v_first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         v_first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None,
+                         v_transposed: bool = False) -> torch.Tensor:
     """proj [T, >= (H + G) D + G Dv]: q heads | k heads | v heads (more columns may follow). Rotates the first
     table.shape[1] coordinates of every q and k head at the token's position (pairs (2i, 2i + 1); `table` as
     `rotation_table` makes it, None: no rotation), divides every head by its root mean square over D, and writes k and
     v of tokens with slot >= 0 into the paged caches; with `v_first` [T, G Dv] (a view with unit column stride) and
-    `lam` (one number) the values become (1 - lam) v + lam v_first first. Returns the queries [T, H, D]."""
+    `lam` (one number) the values become (1 - lam) v + lam v_first first. `v_transposed`: the V pages are
+    [pages, G, Dv, 32] (`alloc_kv_cache`'s layout) instead of [pages, G, 32, Dv]. Returns the queries [T, H, D]."""
     T = proj.shape[0]
-    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[3]
+    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[2 if v_transposed else 3]
     H = n_heads
     R = 0 if table is None else table.shape[1]
     assert proj.stride(1) == 1 and proj.shape[1] >= (H + G) * D + G * V and R <= D and R % 2 == 0
@@ -123,7 +125,8 @@ def rot_norm_cache_write(proj: torch.Tensor, positions: torch.Tensor, table: Opt
             L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(positions), L.ptr(table), L.c_int(table.shape[0]), L.c_int(R),
             L.ptr(slots), L.ptr(v_first), L.c_int64(v_first.stride(0) if v_first is not None else 0), L.ptr(lam),
             L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V),
-            L.c_float(eps), L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "rot_norm_cache_write")
+            L.c_float(eps), L.c_int(int(v_transposed)), L.c_int(L.dtype_flag(proj)), L.stream_ptr()),
+            "rot_norm_cache_write")
         return q
     qk = proj[:, :(H + G) * D].float().view(T, H + G, D)
     if R:
@@ -142,8 +145,56 @@ def rot_norm_cache_write(proj: torch.Tensor, positions: torch.Tensor, table: Opt
     if ok.any():
         pg, off = (slots[ok] // PAGE_SIZE).long(), (slots[ok] % PAGE_SIZE).long()
         kcache[pg, :, off, :] = qk[:, H:][ok].to(kcache.dtype)
-        vcache[pg, :, off, :] = v[ok].view(-1, G, V).to(vcache.dtype)
+        if v_transposed:
+            vcache[pg, :, :, off] = v[ok].view(-1, G, V).to(vcache.dtype)
+        else:
+            vcache[pg, :, off, :] = v[ok].view(-1, G, V).to(vcache.dtype)
     return q
+
+
+def standard_layout_ok(dim: int, vdim: int, dtype, device) -> bool:
+    """Whether an attention layer without head mixing, cap, bias or sink can live in the engine's standard cache
+    (K [pages, G, 32, 128], V transposed) and run its matrix-core flash / paged-decode kernels."""
+    return dim == vdim == 128 and dtype == torch.bfloat16 and torch.device(device).type == "cuda"
+
+
+def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: torch.Tensor, block_tables: torch.Tensor,
+                              cu_q: torch.Tensor, cu_k: torch.Tensor, ctx_len: torch.Tensor, max_q: int,
+                              shape: ScoreShape, nsplit: int = 1,
+                              workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+    """`window_attention` for layers in the standard cache layout (bf16, head size 128, V pages [pages, G, 128, 32]):
+    plain scaled scores behind the window that keeps the first tokens. Prompt portions run the paged flash kernel,
+    single-query rows the paged decode kernel (``csrc/hip/flash_attn_paged.hip``, ``csrc/hip/paged_attn.hip``), both
+    with the softmax weights at 16 bits of mantissa. cu_k int32 [B + 1]: cumulative context lengths."""
+    T, H, D = q.shape
+    G = kcache.shape[1]
+    B = cu_q.numel() - 1
+    assert L.use_hip(q) and q.dtype == torch.bfloat16 and D == 128 and vcache_t.shape[2] == 128 and q.is_contiguous()
+    assert shape.softcap <= 0 and shape.slope_exp == 0 and not shape.sink
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and ctx_len.dtype == torch.int32
+    out = torch.empty(T, H, D, dtype=q.dtype, device=q.device)
+    if max_q == 1:
+        assert T == B
+        pa = pm = None
+        if nsplit > 1:
+            if workspace is None:
+                workspace = (torch.empty(T * nsplit * H * D, dtype=torch.float32, device=q.device),
+                             torch.empty(T * nsplit * H * 2, dtype=torch.float32, device=q.device))
+            pa, pm = workspace
+            assert pa.numel() >= T * nsplit * H * D and pm.numel() >= T * nsplit * H * 2
+        L.check(L.lib().areal_paged_decode_window(
+            L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.ptr(ctx_len), L.ptr(out), L.ptr(pa),
+            L.ptr(pm), L.c_int(B), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(block_tables.shape[1]),
+            L.c_int(int(nsplit)), L.c_float(shape.scale), L.c_int(q.stride(0)), L.c_int(int(shape.window)),
+            L.c_int(int(shape.keep_first)), L.stream_ptr()), "paged_decode_window")
+        return out
+    assert cu_q.dtype == torch.int32 and cu_k.dtype == torch.int32
+    L.check(L.lib().areal_flash_fwd_paged_window(
+        L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(out),
+        L.ptr(cu_q), L.ptr(cu_k), L.c_int(B), L.c_int(int(max_q)), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D),
+        L.c_int64(q.stride(0)), L.c_int64(out.stride(0)), L.c_float(shape.scale), L.c_int(int(shape.window)),
+        L.c_int(int(shape.keep_first)), L.stream_ptr()), "flash_fwd_paged_window")
+    return out
 
 
 def decode_splits(batch: int, window: int, max_context: int, keep_first: int = 0) -> int:

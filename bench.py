@@ -105,9 +105,10 @@ def parse_args():
                         "beside a Qwen3-style transformer of equal size, one JSON line per size; comma-separated names "
                         "out of w1024, w2048, w4096, or 'all' (--prompts-per-gpu prompts of --prompt-len-max tokens, "
                         "--max-new-tokens new tokens each)")
-    p.add_argument("--serve-compare-design", default="kuzanex", choices=["kuzanex", "lufivik"],
-                   help="the layer-list design --serve-compare measures: kuzanex beside a Qwen3-style twin, or lufivik "
-                        "(latent attention, routed experts) beside a Qwen3-MoE-style twin")
+    p.add_argument("--serve-compare-design", default="kuzanex", choices=["kuzanex", "lufivik", "pobelorn"],
+                   help="the layer-list design --serve-compare measures: kuzanex beside a Qwen3-style twin, lufivik "
+                        "(latent attention, routed experts) or pobelorn (parallel blocks, window + lightning "
+                        "attention, routed + shared experts) beside a Qwen3-MoE-style twin")
     a = p.parse_args()
     if a.seq_len:
         a.max_new_tokens = a.seq_len - a.prompt_len_max

@@ -15,18 +15,23 @@
 //     there: their V values are zeroed on the way into LDS (their probabilities are zero, but 0 x NaN is not).
 // Causal masking is aligned bottom-right: query i of a chunk of q_len rows sees keys 0 .. k_len - q_len + i.
 //
+// WIN = true adds a sliding window that keeps the first tokens (a query at position p sees key j <= p when
+// p - j < window or j < keep): key tiles that no query of the workgroup can see are skipped (the tiles that hold kept
+// tokens, then the tiles from the window's start on), and the softmax weights enter O^T += V^T.P^T as the pair
+// (bf16(p), bf16(p - bf16(p))), two products, so that they carry 16 bits of mantissa instead of 8.
+//
 // Role in the reference: prefill against the radix cache inside its serving engine, and
 // flash_attn_with_kvcache at realhf/impl/model/modules/attn.py:272.
 #include "flash_tiles.hpp"
 
 // FP8: the caches hold e4m3 bytes (same layouts): a thread fetches 8 bytes per fragment and widens them to bf16 on the
 // way into LDS; everything behind the staging is the bf16 kernel.
-template <bool FP8>
+template <bool FP8, bool WIN = false>
 __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
     const bf16_t* __restrict__ q, const void* __restrict__ kcache, const void* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, bf16_t* __restrict__ o, float* __restrict__ lse,
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, int64_t q_stride, int64_t o_stride, int Hq, int Hkv,
-    int nbatch, int total_q, float scale_log2, int causal) {
+    int nbatch, int total_q, float scale_log2, int causal, int window = 0, int keep = 0) {
   constexpr int D = 128;
   __shared__ __attribute__((aligned(16))) char smem[2 * 64 * 256];
   char* ks = smem;             // K tile  [64 keys][256 B], 16-byte chunks swizzled (flash_tiles.hpp)
@@ -75,6 +80,14 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
     k_hi = min(k_len, last_q + shift + 1);
   }
   const int ntile_k = k_hi > 0 ? (k_hi + 63) / 64 : 0;
+  // WIN: tiles [0, n_keep) and [t_lo, ntile_k) are walked, `tile_of` maps the step to its tile
+  int t_lo = 0, n_keep = 0;
+  if (WIN && window > 0) {
+    t_lo = min(max(0, qt * 128 + shift - window + 1) / 64, ntile_k);
+    n_keep = min((max(keep, 0) + 63) / 64, t_lo);
+  }
+  const int n_iter = n_keep + ntile_k - t_lo;
+  auto tile_of = [&](int it) { return it < n_keep ? it : t_lo + it - n_keep; };
 
   // K: thread -> (key row = tid>>4 + 16 i, 16-byte chunk tid&15). V^T: piece id = tid + 256 i ->
   // (page half = id>>9, channel = (id>>2)&127, 8-token chunk = id&3): a wave reads 1 KiB of contiguous cache.
@@ -115,16 +128,17 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
       *reinterpret_cast<bf16x4*>(row + (((c8 + 1) ^ sw) << 3)) = hi;
     }
   };
-  if (ntile_k > 0) {
-    load_tile(0);
-    store_tile(0);
+  if (n_iter > 0) {
+    load_tile(tile_of(0));
+    store_tile(tile_of(0));
   }
   __syncthreads();
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): see flash_fwd_kernel
 
   const int vsw = (r >> 1) & 15;  // swizzle key of this lane's V^T rows (32 db + r)
-  for (int t = 0; t < ntile_k; ++t) {
-    if (t + 1 < ntile_k) load_tile(t + 1);
+  for (int it = 0; it < n_iter; ++it) {
+    const int t = tile_of(it);
+    if (it + 1 < n_iter) load_tile(tile_of(it + 1));
     f32x16 sacc[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -141,7 +155,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
       }
     }
     const int kbase = t * 64;
-    const bool need_mask = (kbase + 64 > k_len) || (causal && (kbase + 63 > q0 + shift));
+    const bool windowed = WIN && window > 0;
+    const bool need_mask = (kbase + 64 > k_len) || (causal && (kbase + 63 > q0 + shift)) ||
+                           (windowed && kbase < q0 + 31 + shift - window + 1);
     float mx = -INFINITY;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -151,6 +167,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
         if (need_mask) {
           const int key = kbase + 32 * kb + (j & 3) + 8 * (j >> 2) + 4 * hf;
           if (key >= k_len || (causal && key > my_q + shift)) sv = -INFINITY;
+          if (windowed && my_q + shift - key >= window && key >= keep) sv = -INFINITY;
         }
         sacc[kb][j] = sv;
         mx = fmaxf(mx, sv);
@@ -160,14 +177,16 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
     const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2(m - mn);
     m = mn;
     float ls = 0.f;
-    bf16x8 pf[4];
+    bf16x8 pf[4], pl[WIN ? 4 : 1];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const float pr = (m == -INFINITY) ? 0.f : fast_exp2(sacc[kb][j] - m);
         ls += pr;
-        pf[2 * kb + (j >> 3)][j & 7] = f2bf(pr);
+        const bf16_t ph = f2bf(pr);
+        pf[2 * kb + (j >> 3)][j & 7] = ph;
+        if (WIN) pl[2 * kb + (j >> 3)][j & 7] = f2bf(pr - bf2f(ph));
       }
     l = l * alpha + ls;
     if (__any(alpha != 1.f)) {
@@ -188,10 +207,13 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
         a1[db] = *reinterpret_cast<const bf16x4*>(row + (((4 * s + 2 + hf) ^ vsw) << 3));
       }
 #pragma unroll
-      for (int db = 0; db < 4; ++db) oacc[db] = mfma32(cat4(a0[db], a1[db]), pf[s], oacc[db]);
+      for (int db = 0; db < 4; ++db) {
+        oacc[db] = mfma32(cat4(a0[db], a1[db]), pf[s], oacc[db]);
+        if (WIN) oacc[db] = mfma32(cat4(a0[db], a1[db]), pl[s], oacc[db]);
+      }
     }
     __syncthreads();
-    if (t + 1 < ntile_k) store_tile(t + 1);
+    if (it + 1 < n_iter) store_tile(tile_of(it + 1));
     __syncthreads();
   }
   l = sum_xor32(l);
@@ -234,5 +256,26 @@ extern "C" int areal_flash_fwd_paged(const void* q, const void* kcache, const vo
   else
     hipLaunchKernelGGL(flash_fwd_paged_kernel<false>, grid, block, 0, st, (const bf16_t*)q, kcache, vcache, block_tables,
                        max_pages, (bf16_t*)o, lse, cu_q, cu_k, q_stride, o_stride, Hq, Hkv, B, total_q, scale_log2, causal);
+  return (int)hipGetLastError();
+}
+
+// The same over a sliding window that keeps the first `keep` tokens (window <= 0: every earlier key), bf16 caches,
+// softmax weights at 16 bits of mantissa; always causal.
+extern "C" int areal_flash_fwd_paged_window(const void* q, const void* kcache, const void* vcache,
+                                            const int* block_tables, int max_pages, void* o, const int* cu_q,
+                                            const int* cu_k, int B, int max_q, int total_q, int Hq, int Hkv, int D,
+                                            int64_t q_stride, int64_t o_stride, float softmax_scale, int window, int keep,
+                                            hipStream_t st) {
+  if (B == 0 || max_q == 0) return 0;
+  if (D != 128) return -1;
+  if (Hq % Hkv != 0) return -2;
+  if ((q_stride | o_stride) % 8 != 0) return -3;
+  if (((uintptr_t)q | (uintptr_t)kcache | (uintptr_t)vcache | (uintptr_t)o) % 16 != 0) return -4;
+  const float scale_log2 = softmax_scale * 1.4426950408889634f;
+  const int n_g_pad = (Hkv * B + 7) & ~7;
+  dim3 grid((unsigned)(((max_q + 127) / 128) * (Hq / Hkv) * n_g_pad)), block(256);
+  hipLaunchKernelGGL((flash_fwd_paged_kernel<false, true>), grid, block, 0, st, (const bf16_t*)q, kcache, vcache,
+                     block_tables, max_pages, (bf16_t*)o, (float*)nullptr, cu_q, cu_k, q_stride, o_stride, Hq, Hkv, B,
+                     total_q, scale_log2, 1, window, keep);
   return (int)hipGetLastError();
 }

@@ -29,12 +29,16 @@ DEVINL f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
 // part_o: [B, Hq, nsplit, D] fp32, part_ml: [B, Hq, nsplit, 2] (m in log2 units, l).
 // FP8: the caches hold e4m3 bytes (same layouts); a lane fetches 8 bytes per fragment and widens them to bf16 in
 // registers - half the HBM traffic of the kernel, which is what bounds it at long contexts.
-template <int D, bool FP8>
+// WIN = true: the query (the context's last token) sees key j when ctx - 1 - j < window or j < keep (window <= 0:
+// every key); pages without a visible key are skipped, and the softmax weights enter the P.V product as the pair
+// (bf16(p), bf16(p - bf16(p))) so that they carry 16 bits of mantissa.
+template <int D, bool FP8, bool WIN = false>
 __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
     const bf16_t* __restrict__ q, const void* __restrict__ kcache,
     const void* __restrict__ vcache, const int* __restrict__ block_tables,
     const int* __restrict__ context_lens, bf16_t* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int Hq, int Hkv, int max_pages, float scale_log2, int q_stride) {
+    float* __restrict__ part_ml, int Hq, int Hkv, int max_pages, float scale_log2, int q_stride, int window = 0,
+    int keep = 0) {
   constexpr int KS = D / 32;  // k-steps of the QK product
   constexpr int DB = D / 16;  // 16-wide d blocks of the PV product
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -44,9 +48,14 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
   const int col = lane & 15, c = lane >> 4;
   const int ctx = context_lens[b];
   const int npages = (ctx + PAGE - 1) / PAGE;
-  const int per = (npages + nsplit - 1) / nsplit;
+  // WIN: pages [0, n_keep) and [p_lo, npages) are walked; step i of the walk is page i (i < n_keep) or p_lo + i - n_keep
+  const bool windowed = WIN && window > 0;
+  const int p_lo = windowed ? max(0, ctx - window) / PAGE : 0;
+  const int n_keep = windowed ? min((max(keep, 0) + PAGE - 1) / PAGE, p_lo) : 0;
+  const int nwalk = n_keep + npages - p_lo;
+  const int per = (nwalk + nsplit - 1) / nsplit;
   const int p_beg = split * per;
-  const int p_end = min(npages, p_beg + per);
+  const int p_end = min(nwalk, p_beg + per);
 
   // Q as the B operand of S^T = K.Q^T: lane (q = col, c) holds Q[q][32ks + 8c + j]
   bf16x8 qf[KS];
@@ -63,7 +72,8 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
   float m = -INFINITY, l = 0.f;  // running max (log2 units) is shared by the 4 lanes of a q
 
   const int* bt = block_tables + (size_t)b * max_pages;
-  for (int p = p_beg + wid; p < p_end; p += 4) {
+  for (int pi = p_beg + wid; pi < p_end; pi += 4) {
+    const int p = pi < n_keep ? pi : p_lo + pi - n_keep;
     const int page = bt[p];
     const size_t kp = ((size_t)page * Hkv + h) * PAGE * D;  // element offsets of this page's K / V block
     const size_t vp = ((size_t)page * Hkv + h) * D * PAGE;
@@ -92,7 +102,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const float v = (r < 4 ? sa[r] : sb[r - 4]) * scale_log2;
-      s[r] = (key0 + r < ctx) ? v : -INFINITY;
+      s[r] = (key0 + r < ctx && (!windowed || ctx - 1 - (key0 + r) < window || key0 + r < keep)) ? v : -INFINITY;
       mx = fmaxf(mx, s[r]);
     }
     mx = max_xor16(mx);
@@ -105,18 +115,22 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
       for (int i = 0; i < DB; ++i) o[i] *= alpha;
       m = mn;
     }
-    bf16x8 pf;
+    bf16x8 pf, pl;
     float ls = 0.f;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const float pr = (m == -INFINITY) ? 0.f : fast_exp2(s[r] - m);
       ls += pr;
       pf[r] = f2bf(pr);
+      if (WIN) pl[r] = f2bf(pr - bf2f(pf[r]));
     }
     l += ls;
     // O^T[d, q] += V^T[d, keys] . P^T[keys, q]
 #pragma unroll
-    for (int i = 0; i < DB; ++i) o[i] = mfma16(vt[i], pf, o[i]);
+    for (int i = 0; i < DB; ++i) {
+      o[i] = mfma16(vt[i], pf, o[i]);
+      if (WIN) o[i] = mfma16(vt[i], pl, o[i]);
+    }
   }
   // l is a per-lane partial over this lane's keys: sum the 4 lanes that share a q
   l = sum_xor16(l);
@@ -251,6 +265,30 @@ extern "C" int areal_paged_decode(const void* q, const void* kcache, const void*
   if (nsplit > 1)
     hipLaunchKernelGGL(paged_decode_reduce_kernel, dim3(B * Hq), dim3(D), 0, st, part_o, part_ml,
                        (bf16_t*)out, nsplit, D);
+  return (int)hipGetLastError();
+}
+
+// Decode over a sliding window that keeps the first `keep` tokens; bf16 caches, head sizes 64 / 128.
+extern "C" int areal_paged_decode_window(const void* q, const void* kcache, const void* vcache, const int* block_tables,
+                                         const int* context_lens, void* out, float* part_o, float* part_ml, int B,
+                                         int Hq, int Hkv, int D, int max_pages, int nsplit, float softmax_scale,
+                                         int q_stride, int window, int keep, hipStream_t st) {
+  if (B == 0) return 0;
+  if (Hq % Hkv != 0 || Hq / Hkv > 16) return -1;
+  if (D != 128 && D != 64) return -2;
+  if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -3;
+  const float scale_log2 = softmax_scale * 1.4426950408889634f;
+  const size_t lds = (size_t)(4 * 16 * (D + 4) + 2 * 4 * 16) * sizeof(float);
+  if (D == 128)
+    hipLaunchKernelGGL((paged_decode_kernel<128, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
+                       (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
+                       Hkv, max_pages, scale_log2, q_stride, window, keep);
+  else
+    hipLaunchKernelGGL((paged_decode_kernel<64, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
+                       (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
+                       Hkv, max_pages, scale_log2, q_stride, window, keep);
+  if (nsplit > 1)
+    hipLaunchKernelGGL(paged_decode_reduce_kernel, dim3(B * Hq), dim3(D), 0, st, part_o, part_ml, (bf16_t*)out, nsplit, D);
   return (int)hipGetLastError();
 }
 

@@ -83,7 +83,7 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
     const T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ table,
     int n_pos, int R, const int64_t* __restrict__ slots, const T* __restrict__ v_first, int64_t vf_stride,
     const T* __restrict__ lam_p, T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache, int H, int G,
-    int D, int V, float eps) {
+    int D, int V, float eps, int v_transposed) {
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * row_stride;
   const int64_t slot = slots[t];
@@ -129,7 +129,8 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
       const int c = i / V, v = i % V;
       float x = ldf<T>(vsrc, i);
       if (v_first) x = (1.f - lam) * x + lam * ldf<T>(v_first, (size_t)t * vf_stride + i);
-      stf<T>(vcache, ((page * G + c) * PAGE + off) * V + v, x);
+      // V pages are [G][32][V], or [G][V][32] (a channel's 32 tokens side by side) for the kernels that want V^T
+      stf<T>(vcache, v_transposed ? ((page * G + c) * V + v) * PAGE + off : ((page * G + c) * PAGE + off) * V + v, x);
     }
   }
 }
@@ -308,8 +309,8 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// Matrix-core version for bf16 prompt portions (head sizes 64 / 128, up to 16 heads). One workgroup = 16 queries x
-// all heads, H / HPW waves, wave w owning heads w HPW .. w HPW + HPW - 1. Per 32-key page:
+// Matrix-core version for bf16 prompt portions (head sizes 64 / 128). One workgroup = 16 queries x all heads (up to 16;
+// without head mixing more heads are split into groups of whole key/value heads over grid z), H / HPW waves, wave w owning heads w HPW .. w HPW + HPW - 1. Per 32-key page:
 //   stage   K of every key/value head -> LDS [G][32][D + 8], V transposed -> LDS [G][V][32 + 8]
 //   scores  per owned head: q (registers) x K^T, bf16 MFMA 16x16x32 with fp32 accumulation; scale, cap, distance bias
 //           in fp32 -> LDS SM[head][query][key] (fp32)
@@ -323,9 +324,12 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const bf16_t* __restrict__ mix, const bf16_t* __restrict__ gate,
-    int64_t gate_stride, bf16_t* __restrict__ out, int H, int G, float scale, float softcap, float slope_exp,
-    int window, int keep, int sink) {
+    int64_t gate_stride, bf16_t* __restrict__ out, int Hall, int Gall, int H, float scale, float softcap,
+    float slope_exp, int window, int keep, int sink) {
   constexpr int D = DK * 32, V = VT_ * 16, KS = D + 8, VS = PAGE + 8, SS = PAGE + 4;
+  // this workgroup's heads: hbase .. hbase + H - 1 of Hall (several groups only without head mixing), and their G
+  // key/value heads from c0 on
+  const int rep = Hall / Gall, hbase = blockIdx.z * H, c0 = hbase / rep, G = H / rep;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   unsigned* SM = reinterpret_cast<unsigned*>(smem);                      // [16][16][SS] 4-byte slots
   bf16_t* KT = reinterpret_cast<bf16_t*>(smem + 16 * 16 * SS * 4);       // [G][32][KS]
@@ -337,9 +341,10 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthr = blockDim.x, NW = nthr >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
   const int b = blockIdx.y;
+
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0, t0 = blockIdx.x * 16;
   if (t0 >= qlen) return;
-  const int nq = min(16, qlen - t0), ctx = ctx_len[b], pos0 = ctx - qlen + t0, rep = H / G;
+  const int nq = min(16, qlen - t0), ctx = ctx_len[b], pos0 = ctx - qlen + t0;
 
   for (int i = tid; i < 16 * 16 * SS; i += nthr) SM[i] = 0u;
   for (int i = tid; i < 256; i += nthr) {
@@ -355,10 +360,10 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
 #pragma unroll
   for (int hh = 0; hh < HPW; ++hh) {
     const int h = wave * HPW + hh;
-    slope[hh] = slope_exp != 0.f ? exp2f(-slope_exp * (float)(h + 1) / (float)H) : 0.f;
+    slope[hh] = slope_exp != 0.f ? exp2f(-slope_exp * (float)(hbase + h + 1) / (float)Hall) : 0.f;
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks) {
-      if (r16 < nq) qf[hh][ks] = ld8(q + ((size_t)(q0 + t0 + r16) * H + h) * D + 32 * ks + 8 * quad);
+      if (r16 < nq) qf[hh][ks] = ld8(q + ((size_t)(q0 + t0 + r16) * Hall + hbase + h) * D + 32 * ks + 8 * quad);
       else qf[hh][ks] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
@@ -377,11 +382,11 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
     __syncthreads();  // the page before is consumed (first time: the set-up above is visible)
     for (int i = tid; i < G * PAGE * (D / 8); i += nthr) {
       const int dv = i % (D / 8), key = (i / (D / 8)) % PAGE, c = i / (PAGE * (D / 8));
-      st8(KT + ((size_t)c * PAGE + key) * KS + 8 * dv, ld8(kcache + ((page * G + c) * PAGE + key) * D + 8 * dv));
+      st8(KT + ((size_t)c * PAGE + key) * KS + 8 * dv, ld8(kcache + ((page * Gall + c0 + c) * PAGE + key) * D + 8 * dv));
     }
     for (int i = tid; i < G * PAGE * (V / 8); i += nthr) {
       const int key = i % PAGE, vv = (i / PAGE) % (V / 8), c = i / (PAGE * (V / 8));
-      bf16x8 x = ld8(vcache + ((page * G + c) * PAGE + key) * V + 8 * vv);
+      bf16x8 x = ld8(vcache + ((page * Gall + c0 + c) * PAGE + key) * V + 8 * vv);
       const bool live = jb + key < j_hi;  // rows past the tile's last key may hold anything: they must not reach p.v
 #pragma unroll
       for (int e = 0; e < 8; ++e) VTt[((size_t)c * V + 8 * vv + e) * VS + key] = live ? x[e] : (bf16_t)0.f;
@@ -491,9 +496,9 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
       const size_t tok = (size_t)(q0 + t0 + qi);
       const float l = lS[h * 16 + qi];
       float f = l > 0.f ? 1.f / l : 0.f;
-      if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + h]));
+      if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + hbase + h]));
 #pragma unroll
-      for (int vt = 0; vt < VT_; ++vt) out[(tok * H + h) * V + 16 * vt + r16] = f2bf(acc[hh][vt][i] * f);
+      for (int vt = 0; vt < VT_; ++vt) out[(tok * Hall + hbase + h) * V + 16 * vt + r16] = f2bf(acc[hh][vt][i] * f);
     }
   }
 }
@@ -502,17 +507,28 @@ size_t mfma_lds_bytes(int G, int D, int V) {
   return (size_t)16 * 16 * (PAGE + 4) * 4 + (size_t)G * PAGE * (D + 8) * 2 + (size_t)G * V * (PAGE + 8) * 2 + 4 * 256 * 4;
 }
 int mfma_heads_per_wave(int H) { return (H % 4 == 0 && H >= 16) ? 4 : ((H % 2 == 0 && H >= 8) ? 2 : 1); }
-bool mfma_usable(int H, int G, int D, int V) {
-  if (H > 16 || H < 1 || G < 1 || H % G != 0 || (D != 64 && D != 128) || (V != 32 && V != 64 && V != 128)) return false;
-  if (H / mfma_heads_per_wave(H) > 8) return false;
-  return mfma_lds_bytes(G, D, V) <= 160 * 1024;
+// Heads per workgroup: all of them when the heads' scores are mixed; otherwise the largest group of at most 16 heads
+// that holds whole key/value heads and divides the head count (0: none).
+int mfma_head_group(int H, int G, bool mixed) {
+  if (H < 1 || G < 1 || H % G != 0) return 0;
+  if (mixed || H <= 16) return H <= 16 ? H : 0;
+  const int rep = H / G;
+  for (int hb = 16; hb >= 1; --hb)
+    if (H % hb == 0 && hb % rep == 0) return hb;
+  return 0;
+}
+bool mfma_usable(int H, int G, int D, int V, bool mixed) {
+  if ((D != 64 && D != 128) || (V != 32 && V != 64 && V != 128)) return false;
+  const int hb = mfma_head_group(H, G, mixed);
+  if (hb < 1 || hb / mfma_heads_per_wave(hb) > 8) return false;
+  return mfma_lds_bytes(hb / (H / G), D, V) <= 160 * 1024;
 }
 
 template <int HPW, int MAXT>
 int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* kc, const bf16_t* vc,
                 const int* bt, int max_pages, const int* cu_q, const int* ctx_len, const bf16_t* mix,
-                const bf16_t* gate, int64_t gate_stride, bf16_t* out, int H, int G, int D, int V, float scale,
-                float softcap, float slope_exp, int window, int keep, int sink) {
+                const bf16_t* gate, int64_t gate_stride, bf16_t* out, int Hall, int Gall, int H, int D, int V,
+                float scale, float softcap, float slope_exp, int window, int keep, int sink) {
 #define MFMA_CASE(DKV, VTV)                                                                                        \
   do {                                                                                                             \
     static bool raised = false; /* once per kernel: no attribute call inside a stream capture later */            \
@@ -522,8 +538,8 @@ int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q
       raised = true;                                                                                               \
     }                                                                                                              \
     hipLaunchKernelGGL((window_attn_mfma_kernel<HPW, DKV, VTV, MAXT>), grid, dim3(nthr), lds, st, q, kc, vc, bt,   \
-                       max_pages, cu_q, ctx_len, mix, gate, gate_stride, out, H, G, scale, softcap, slope_exp,     \
-                       window, keep, sink);                                                                        \
+                       max_pages, cu_q, ctx_len, mix, gate, gate_stride, out, Hall, Gall, H, scale, softcap,       \
+                       slope_exp, window, keep, sink);                                                             \
   } while (0)
   if (D == 64 && V == 32) MFMA_CASE(2, 2);
   else if (D == 64 && V == 64) MFMA_CASE(2, 4);
@@ -579,17 +595,17 @@ extern "C" int areal_qk_norm_cache_write(const void* proj, int64_t row_stride, c
 extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, const int* positions, const float* table,
                                           int n_pos, int R, const int64_t* slots, const void* v_first, int64_t vf_stride,
                                           const void* lam, void* q_out, void* kcache, void* vcache, int T, int H, int G,
-                                          int D, int V, float eps, int dt, hipStream_t st) {
+                                          int D, int V, float eps, int v_transposed, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (R < 0 || R > D || R % 2 != 0 || n_pos < 1 || (v_first && !lam)) return -1;
   if (dt == 0)
     hipLaunchKernelGGL(rot_norm_cache_write_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
                        positions, table, n_pos, R, slots, (const bf16_t*)v_first, vf_stride, (const bf16_t*)lam,
-                       (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps);
+                       (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_transposed);
   else
     hipLaunchKernelGGL(rot_norm_cache_write_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
                        positions, table, n_pos, R, slots, (const float*)v_first, vf_stride, (const float*)lam,
-                       (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps);
+                       (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps, v_transposed);
   return (int)hipGetLastError();
 }
 
@@ -611,14 +627,15 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
                                  int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1) return -1;
-  if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(H, G, D, V)) {
-    const int hpw = mfma_heads_per_wave(H), nthr = 64 * (H / hpw);
-    const dim3 mgrid((max_q + 15) / 16, B, 1);
-    const size_t mlds = mfma_lds_bytes(G, D, V);
+  if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(H, G, D, V, mix != nullptr)) {
+    const int hb = mfma_head_group(H, G, mix != nullptr);
+    const int hpw = mfma_heads_per_wave(hb), nthr = 64 * (hb / hpw);
+    const dim3 mgrid((max_q + 15) / 16, B, H / hb);
+    const size_t mlds = mfma_lds_bytes(hb / (H / G), D, V);
 #define MFMA_ARGS                                                                                                  \
   mgrid, nthr, mlds, st, (const bf16_t*)q, (const bf16_t*)kcache, (const bf16_t*)vcache, block_tables, max_pages,   \
-      cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, G, D, V, scale, softcap, \
-      slope_exp, window, keep, sink
+      cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, G, hb, D, V, scale,      \
+      softcap, slope_exp, window, keep, sink
     if (hpw == 4) return launch_mfma<4, 256>(MFMA_ARGS);
     if (hpw == 2) return launch_mfma<2, 512>(MFMA_ARGS);
     return launch_mfma<1, 512>(MFMA_ARGS);

@@ -190,12 +190,20 @@ def _attention_case(H, G, D, V, window, keep, scale, n, probes, seed, rot=None):
     return h, w, m
 
 
-def _run_attention(h, m, dtype, device, portions, pages, nsplit=1, matrix_cores=True):
-    """The ops over a paged cache, the sequence fed in portions; returns [n, H V]."""
+def _run_attention(h, m, dtype, device, portions, pages, nsplit=1, matrix_cores=True, standard=False):
+    """The ops over a paged cache, the sequence fed in portions; returns [n, H V]. `standard`: the cache in the
+    engine's standard layout and its flash / paged-decode kernels (bf16 heads of 128 on the GPU)."""
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     rot = m.get("rot")
     n = h.shape[0]
-    kc, vc = _paged(max(pages) + 2, G, D, V, dtype, device, fill=50.0)
+    if standard:
+        from areal_vllm_amd.ops.attention import alloc_kv_cache
+
+        kc, vc = alloc_kv_cache(max(pages) + 2, G, D, dtype, device)
+        kc.fill_(50.0)
+        vc.fill_(-50.0)
+    else:
+        kc, vc = _paged(max(pages) + 2, G, D, V, dtype, device, fill=50.0)
     table = wattn.rotation_table(rot["base"], rot["dims"], n + 1, device, rot.get("scaling")) if rot else None
     shape = wattn.ScoreShape(scale=m["scale"], window=m["mask"]["size"], keep_first=m["mask"]["keep_first"])
     bt = torch.tensor([pages], dtype=torch.int32, device=device)
@@ -206,9 +214,13 @@ def _run_attention(h, m, dtype, device, portions, pages, nsplit=1, matrix_cores=
         if c <= 0:
             break
         q = wattn.rot_norm_cache_write(hd[at:at + c], i32(list(range(at, at + c)), device), table,
-                                       _slots(pages, at, at + c, device), kc, vc, H, 1e-6)
-        o = wattn.window_attention(q, kc, vc, bt, i32([0, c], device), i32([at + c], device), c, shape, None,
-                                   nsplit=nsplit if c == 1 else 1, matrix_cores=matrix_cores)
+                                       _slots(pages, at, at + c, device), kc, vc, H, 1e-6, v_transposed=standard)
+        if standard:
+            o = wattn.window_attention_standard(q, kc, vc, bt, i32([0, c], device), i32([0, at + c], device),
+                                                i32([at + c], device), c, shape, nsplit=nsplit if c == 1 else 1)
+        else:
+            o = wattn.window_attention(q, kc, vc, bt, i32([0, c], device), i32([at + c], device), c, shape, None,
+                                       nsplit=nsplit if c == 1 else 1, matrix_cores=matrix_cores)
         outs.append(o.reshape(c, H * V).float().cpu())
         at += c
     return torch.cat(outs)
@@ -329,6 +341,46 @@ def test_routed_and_shared_experts(device, dtype, W, ff, E, top, shared):
         with torch.no_grad():
             got = mod(cols, hd, hd.float())
         assert rows_agree(got.float().cpu(), want, dtype), rel_err(got.float().cpu(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,window,keep", [(4, 2, 70, 5), (2, 1, 64, 70), (4, 4, 200, 0), (2, 2, 0, 0), (3, 1, 1, 1)])
+def test_standard_cache_layout_kernels_window_edges_and_portions(H, G, window, keep):
+    """bf16 heads of 128: the engine's paged flash and paged decode kernels behind the window that keeps the first
+    tokens; key tiles of 64, query blocks of 128, pages of 32 and the window's and the kept tokens' edges all fall
+    inside the sequence."""
+    device, dtype, D, n = "cuda", torch.bfloat16, 128, 330
+    assert wattn.standard_layout_ok(D, D, dtype, device) and not wattn.standard_layout_ok(D, 64, dtype, device)
+    w_eff = window if window > 0 else n
+    pages = [3, 1, 4, 9, 2, 11, 7, 5, 8, 6, 10]
+    for k, qi in enumerate((n - 1, 300, 257, 256, 200, 129, 128, 127, 70, 64, 63)):
+        for kj in (qi - w_eff + 1, qi - w_eff, keep - 1, keep, 1, qi - 63, qi - 64, qi - 65):
+            if not 0 <= kj <= qi:
+                continue
+            h, w, m = _attention_case(H, G, D, D, window, keep, 1.0, n, [(qi, kj)], 3 + k)
+            h = h.to(dtype).float()
+            want, _ = O.attention_mixer(h.to(F64)[:qi + 1], w, m, 1e-6, None)
+            for portions, nsplit in (([n], 1), ([qi, 1, n], 1), ([qi, 1, n], 3), ([max(qi - 130, 1), 131, n], 1)):
+                got = _run_attention(h, m, dtype, device, portions, pages, nsplit, standard=True)
+                assert rel_err(got[qi:qi + 1], want[qi:qi + 1]) < tol(dtype), (qi, kj, portions, nsplit)
+    h, w, m = _attention_case(H, G, D, D, window, keep, 0.1, n, [], 1, rot=ROTS[1])
+    h = h.to(dtype).float()
+    want, _ = O.attention_mixer(h.to(F64), w, m, 1e-6, None)
+    for portions in ([n], [1], [2], [3, 127, 1, 1, 64, 131, 2]):
+        got = _run_attention(h, m, dtype, device, portions + [portions[-1]] * n, pages, 2, standard=True)
+        assert rel_err(got, want) < tol(dtype), portions
+
+
+@pytest.mark.parametrize("device,dtype", OP_CASES)
+def test_many_heads_without_mixing_run_in_groups(device, dtype):
+    """More heads than one workgroup of the matrix-core kernel holds: groups of whole key/value heads."""
+    H, G, D, V, n = 32, 8, 64, 32, 70
+    h, w, m = _attention_case(H, G, D, V, 40, 3, 0.3, n, [], 2)
+    if dtype == torch.bfloat16:
+        h = h.to(dtype).float()
+    want, _ = O.attention_mixer(h.to(F64), w, m, 1e-6, None)
+    for portions in ([n], [33, 1, 36]):
+        assert rel_err(_run_attention(h, m, dtype, device, portions, [2, 0, 1]), want) < tol(dtype)
 
 
 # ------------------------------------------------------------------------------------ whole models through the engine
@@ -513,6 +565,9 @@ SHAPES = [
     config([attn(4, 2, 64, 64, 40, 4, 32, ff=64, experts=4, top=2, shared=64), light(2, 64, 64, (0.9, 0.99), ff=128),
             attn(8, 2, 128, 32, 70, 33, 64, v_mix=False, mlp="dense", ff=128), light(1, 128, 128, (0.97,), mlp=None),
             attn(4, 2, 128, 64, 50, 0, 128, mlp=None)], width=64),
+    # heads of 128 for keys and values: in bf16 on the GPU these layers live in the engine's standard cache layout
+    config([attn(4, 2, 128, 128, 40, 4, 64, mlp="dense", ff=64), attn(4, 2, 128, 128, 70, 33, 128, mlp=None),
+            light(2, 32, 32, (0.9, 0.99), mlp=None), attn(2, 2, 128, 128, 0, 0, 32, v_mix=False)], width=64),
 ]
 
 
@@ -603,9 +658,7 @@ def test_config_reader_and_checkpoint_save_then_load(tmp_path):
     m = build_model(cfg, dtype=torch.float32)
     m.flatten()
     m.init_weights(seed=4)
-    # every attention layer carries its mixing number; the ones that never read it are not counted
-    unused = sum(1 for b in m.layers if b.kind == "attention" and b.mix.v_mix != "mix")
-    assert sum(p.numel() for p in m.parameters()) == cfg.n_params() + unused
+    assert sum(p.numel() for p in m.parameters()) == cfg.n_params()  # every attention layer carries a mixing number
     assert [b.mix.v_mix for b in m.layers if b.kind == "attention"] == ["first", "mix", None]
     m.save_checkpoint(str(tmp_path))
     cfg2 = ModelConfig.from_pretrained(str(tmp_path))
