@@ -588,10 +588,8 @@ class RoutedSwiGLUExperts(nn.Module):
         return 2 * self.shared_ff
 
     def forward(self, cols: torch.Tensor, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
-        if hc.dtype == torch.float32:
-            z = F.linear(hc, self.router, self.router_bias)
-        else:  # fp32 products on the norm's fp32 output when there is one, else on its rounding
-            z = F.linear(h32 if h32 is not None else hc.float(), self.router.float(), self.router_bias.float())
+        # fp32 products on the norm's fp32 output when there is one, else on its rounding
+        z = pblock.router_logits(h32 if h32 is not None else hc.float(), self.router, self.router_bias)
         # softmax over all logits, the k largest re-normalised: the softmax over the chosen logits
         topv, topi = moe_ops.moe_topk(z, self.k, True, out_dtype=torch.float32)
         order, inv, src_row, offsets = moe_ops.moe_sort(topi.reshape(-1), self.E, self.k)

@@ -84,3 +84,19 @@ def relu2_rows(z: torch.Tensor) -> torch.Tensor:
                                          L.c_int(L.dtype_flag(z)), L.stream_ptr()), "relu2_rows")
         return out
     return torch.relu(z.float()).pow(2).to(z.dtype)
+
+
+def router_logits(h32: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """z = h32 W^T + b in fp32: h32 fp32 [T, W] (a norm's fp32 output), weight [E, W] and bias [E] in the model's
+    dtype (read as they are, products and sums in fp32)."""
+    T, W = h32.shape
+    E = weight.shape[0]
+    assert h32.dtype == torch.float32
+    if L.use_hip(h32):
+        assert h32.is_contiguous() and weight.is_contiguous() and weight.shape == (E, W)
+        assert bias is None or (bias.dtype == weight.dtype and bias.numel() == E)
+        z = torch.empty(T, E, dtype=torch.float32, device=h32.device)
+        L.check(L.lib().areal_router_logits(L.ptr(h32), L.ptr(weight), L.ptr(bias), L.ptr(z), L.c_int(T), L.c_int(W),
+                                            L.c_int(E), L.c_int(L.dtype_flag(weight)), L.stream_ptr()), "router_logits")
+        return z
+    return F.linear(h32, weight.float(), bias.float() if bias is not None else None)

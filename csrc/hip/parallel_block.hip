@@ -45,6 +45,56 @@ __global__ void __launch_bounds__(256) sum_norm_kernel(float* __restrict__ x, co
   }
 }
 
+template <typename T> DEVINL f32x4 ld4(const T* p, size_t i);
+template <> DEVINL f32x4 ld4<bf16_t>(const bf16_t* p, size_t i) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p + i);
+  return (f32x4){bf2f(v[0]), bf2f(v[1]), bf2f(v[2]), bf2f(v[3])};
+}
+template <> DEVINL f32x4 ld4<float>(const float* p, size_t i) { return *reinterpret_cast<const f32x4*>(p + i); }
+template <typename T> DEVINL void st4(T* p, size_t i, f32x4 v);
+template <> DEVINL void st4<bf16_t>(bf16_t* p, size_t i, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p + i) = (bf16x4){f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+}
+template <> DEVINL void st4<float>(float* p, size_t i, f32x4 v) { *reinterpret_cast<f32x4*>(p + i) = v; }
+
+// The same for rows of up to 1024 NV elements that are multiples of 4: the row stays in registers between the sum of
+// squares and the scaling, and moves as 8- / 16-byte vectors.
+template <typename T, int NV>
+__global__ void __launch_bounds__(256) sum_norm_vec_kernel(float* __restrict__ x, const T* __restrict__ y1,
+                                                            const T* __restrict__ y2, const T* __restrict__ w,
+                                                            float* __restrict__ o32, T* __restrict__ oc, int W, float eps) {
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * W;
+  f32x4 z[NV];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < W) {
+      z[v] = *reinterpret_cast<const f32x4*>(x + base + i);
+      if (y1) {
+        z[v] += ld4<T>(y1, base + i);
+        if (y2) z[v] += ld4<T>(y2, base + i);
+        *reinterpret_cast<f32x4*>(x + base + i) = z[v];
+      }
+      ss += z[v][0] * z[v][0] + z[v][1] * z[v][1] + z[v][2] * z[v][2] + z[v][3] * z[v][3];
+    }
+  }
+  if (!w) return;
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int i = 4 * (threadIdx.x + 256 * v);
+    if (i < W) {
+      // the weight may sit anywhere in a flat parameter buffer: element loads
+      const f32x4 h = z[v] * r * (f32x4){ldf<T>(w, i), ldf<T>(w, i + 1), ldf<T>(w, i + 2), ldf<T>(w, i + 3)};
+      if (o32) *reinterpret_cast<f32x4*>(o32 + base + i) = h;
+      if (oc) st4<T>(oc, base + i, h);
+    }
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) embed_scale_kernel(const int64_t* __restrict__ tokens, const T* __restrict__ embed,
                                                            float* __restrict__ out, int W, int vocab, float scale) {
@@ -80,6 +130,31 @@ __global__ void __launch_bounds__(256) relu2_rows_kernel(const T* __restrict__ z
   }
 }
 
+// z[t, e] = x[t, :] . w[e, :] + b[e]: fp32 input rows (a norm's fp32 output), weights in the storage type, fp32 sums. A
+// workgroup takes GT tokens and four weight rows (one a wave), so a weight row is read once per GT tokens.
+template <typename T, int GT>
+__global__ void __launch_bounds__(256) router_logits_kernel(const float* __restrict__ x, const T* __restrict__ w,
+                                                             const T* __restrict__ bias, float* __restrict__ z, int Ttok,
+                                                             int W, int E) {
+  const int t0 = blockIdx.x * GT, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int u = blockIdx.y * 4 + wave;
+  if (u >= E) return;
+  const T* wr = w + (size_t)u * W;
+  float s[GT];
+#pragma unroll
+  for (int tt = 0; tt < GT; ++tt) s[tt] = 0.f;
+  for (int i = lane; i < W; i += 64) {
+    const float wv = ldf<T>(wr, i);
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) s[tt] += x[(size_t)min(t0 + tt, Ttok - 1) * W + i] * wv;
+  }
+#pragma unroll
+  for (int tt = 0; tt < GT; ++tt) {
+    const float tot = wave_sum(s[tt]);
+    if (lane == 0 && t0 + tt < Ttok) z[(size_t)(t0 + tt) * E + u] = tot + (bias ? ldf<T>(bias, u) : 0.f);
+  }
+}
+
 int blocks_for(int64_t total) { return (int)((total + 255) / 256 < 65535 * 8 ? (total + 255) / 256 : 65535 * 8); }
 
 }  // namespace
@@ -89,6 +164,22 @@ extern "C" int areal_sum_norm(float* x, const void* y1, const void* y2, const vo
                               float eps, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (y2 && !y1) return -1;
+  if (W % 4 == 0 && W <= 4096) {
+#define VEC(TT, NVV)                                                                                                \
+  hipLaunchKernelGGL((sum_norm_vec_kernel<TT, NVV>), dim3(T), dim3(256), 0, st, x, (const TT*)y1, (const TT*)y2,     \
+                     (const TT*)w, o32, (TT*)oc, W, eps)
+    if (dt == 0) {
+      if (W <= 1024) VEC(bf16_t, 1);
+      else if (W <= 2048) VEC(bf16_t, 2);
+      else VEC(bf16_t, 4);
+    } else {
+      if (W <= 1024) VEC(float, 1);
+      else if (W <= 2048) VEC(float, 2);
+      else VEC(float, 4);
+    }
+#undef VEC
+    return (int)hipGetLastError();
+  }
   if (dt == 0)
     hipLaunchKernelGGL(sum_norm_kernel<bf16_t>, dim3(T), dim3(256), 0, st, x, (const bf16_t*)y1, (const bf16_t*)y2,
                        (const bf16_t*)w, o32, (bf16_t*)oc, W, eps);
@@ -132,5 +223,23 @@ extern "C" int areal_relu2_rows(const void* z, int64_t row_stride, void* out, in
   else
     hipLaunchKernelGGL(relu2_rows_kernel<float>, dim3(nb), dim3(256), 0, st, (const float*)z, row_stride, (float*)out, n,
                        F);
+  return (int)hipGetLastError();
+}
+
+// x fp32 [T, W], w [E, W] and bias [E] (or null) in the storage type -> z fp32 [T, E]
+extern "C" int areal_router_logits(const float* x, const void* w, const void* bias, float* z, int T, int W, int E, int dt,
+                                   hipStream_t st) {
+  if (T == 0 || E == 0) return 0;
+#define LAUNCH(TT, GTV)                                                                                              \
+  hipLaunchKernelGGL((router_logits_kernel<TT, GTV>), dim3((T + GTV - 1) / GTV, (E + 3) / 4), dim3(256), 0, st, x,   \
+                     (const TT*)w, (const TT*)bias, z, T, W, E)
+  if (dt == 0) {
+    if (T < 512) LAUNCH(bf16_t, 1);
+    else LAUNCH(bf16_t, 8);
+  } else {
+    if (T < 512) LAUNCH(float, 1);
+    else LAUNCH(float, 8);
+  }
+#undef LAUNCH
   return (int)hipGetLastError();
 }

@@ -93,7 +93,8 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
   const int pos = min(max(positions[t], 0), n_pos - 1);
   const float* cs = table + (size_t)pos * R;
   const int half = R / 2;
-  for (int u = wave; u < H + G; u += 4) {
+  // grid y spreads a token's heads over workgroups (one head a wave when there are enough of them)
+  for (int u = blockIdx.y * 4 + wave; u < H + G; u += 4 * gridDim.y) {
     if (u >= H && slot < 0) continue;
     const T* src = row + (size_t)u * D;
     T* dst = u < H ? q_out + ((size_t)t * H + u) * D : kcache + ((page * G + (u - H)) * PAGE + off) * D;
@@ -125,7 +126,7 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
   if (slot >= 0) {
     const T* vsrc = row + (size_t)(H + G) * D;
     const float lam = v_first ? ldf<T>(lam_p, 0) : 0.f;
-    for (int i = threadIdx.x; i < G * V; i += 256) {
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < G * V; i += 256 * gridDim.y) {
       const int c = i / V, v = i % V;
       float x = ldf<T>(vsrc, i);
       if (v_first) x = (1.f - lam) * x + lam * ldf<T>(v_first, (size_t)t * vf_stride + i);
@@ -598,12 +599,14 @@ extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, 
                                           int D, int V, float eps, int v_transposed, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (R < 0 || R > D || R % 2 != 0 || n_pos < 1 || (v_first && !lam)) return -1;
+  // few tokens (decoding): a head a wave; many: a token a workgroup
+  const dim3 grid(T, T <= 512 ? (H + G + 3) / 4 : 1);
   if (dt == 0)
-    hipLaunchKernelGGL(rot_norm_cache_write_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
+    hipLaunchKernelGGL(rot_norm_cache_write_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)proj, row_stride,
                        positions, table, n_pos, R, slots, (const bf16_t*)v_first, vf_stride, (const bf16_t*)lam,
                        (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_transposed);
   else
-    hipLaunchKernelGGL(rot_norm_cache_write_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
+    hipLaunchKernelGGL(rot_norm_cache_write_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, row_stride,
                        positions, table, n_pos, R, slots, (const float*)v_first, vf_stride, (const float*)lam,
                        (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps, v_transposed);
   return (int)hipGetLastError();
