@@ -86,13 +86,17 @@ def relu2_rows(z: torch.Tensor) -> torch.Tensor:
     return torch.relu(z.float()).pow(2).to(z.dtype)
 
 
+ROUTER_KERNEL_MAX_ROWS = 256
+
+
 def router_logits(h32: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     """z = h32 W^T + b in fp32: h32 fp32 [T, W] (a norm's fp32 output), weight [E, W] and bias [E] in the model's
-    dtype (read as they are, products and sums in fp32)."""
+    dtype (read as they are, products and sums in fp32). Few rows (decoding) run one wave per (row, expert); many rows
+    the fp32 library product."""
     T, W = h32.shape
     E = weight.shape[0]
     assert h32.dtype == torch.float32
-    if L.use_hip(h32):
+    if L.use_hip(h32) and T <= ROUTER_KERNEL_MAX_ROWS:
         assert h32.is_contiguous() and weight.is_contiguous() and weight.shape == (E, W)
         assert bias is None or (bias.dtype == weight.dtype and bias.numel() == E)
         z = torch.empty(T, E, dtype=torch.float32, device=h32.device)

@@ -143,20 +143,74 @@ __global__ void __launch_bounds__(256) lightning_chunk_kernel(
     for (int j = tid; j <= CL; j += 256) pw[j] = j == 0 ? 1.f : exp2f((float)j * l2);
   }
 
+  // 16-byte loads of a chunk's operands, fetched into registers one chunk ahead so that their latency runs under the
+  // matrix work of the chunk before (rows and offsets that are multiples of a vector, key size = its padded size)
+  constexpr int VE = 16 / (int)sizeof(T);                 // elements per vector
+  constexpr int NKQ = CL * DP / VE / 256;                 // vectors per thread of K (and of Q)
+  constexpr int NVV = CL * 64 / VE / 256;                 // vectors per thread of V
+  const bool vec = D == DP && row_stride % VE == 0 && q_off % VE == 0 && k_off % VE == 0 && v_off % VE == 0 &&
+                   V % VE == 0 && (reinterpret_cast<uintptr_t>(proj) & 15) == 0;
+  u32x4 rk[NKQ], rq[NKQ], rv[NVV];
+  auto fetch = [&](int tb) {
+    const int nt = min(CL, t_hi - tb);
+#pragma unroll
+    for (int j = 0; j < NKQ; ++j) {
+      const int e = (tid + 256 * j) * VE, d = e % DP, tt = e / DP;
+      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+      rk[j] = *reinterpret_cast<const u32x4*>(row + k_off + hd * D + d);
+      rq[j] = *reinterpret_cast<const u32x4*>(row + q_off + hd * D + d);
+    }
+#pragma unroll
+    for (int j = 0; j < NVV; ++j) {
+      const int e = (tid + 256 * j) * VE, c = e % 64, tt = e / 64;
+      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+      rv[j] = (col0 + c < V) ? *reinterpret_cast<const u32x4*>(row + v_off + hd * V + col0 + c) : (u32x4){0u, 0u, 0u, 0u};
+    }
+  };
+  auto unpack = [&](u32x4 r, float* dst, bool live) {  // VE activated values (zeros for rows past the chunk's end)
+    if (sizeof(T) == 2) {
+      const bf16x8 x = __builtin_bit_cast(bf16x8, r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[e] = live ? act_in(bf2f(x[e]), act) : 0.f;
+    } else {
+      const f32x4 x = __builtin_bit_cast(f32x4, r);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[e] = live ? act_in(x[e], act) : 0.f;
+    }
+  };
+  if (vec) fetch(t_lo);
+
   for (int tb = t_lo; tb < t_hi; tb += CL) {
     const int nt = min(CL, t_hi - tb);
     __syncthreads();  // the chunk before is done with the staged operands
-    for (int i = tid; i < CL * DP; i += 256) {
-      const int d = i % DP, tt = i / DP;
-      const bool live = tt < nt && d < D;
-      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
-      Ks[tt * QS + d] = live ? act_in(ldf<T>(row, k_off + hd * D + d), act) : 0.f;
-      Qs[tt * QS + d] = live ? act_in(ldf<T>(row, q_off + hd * D + d), act) : 0.f;
-    }
-    for (int i = tid; i < CL * 64; i += 256) {
-      const int c = i % 64, tt = i / 64;
-      Vs[tt * CS + c] = (tt < nt && col0 + c < V)
-                            ? act_in(ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col0 + c), act) : 0.f;
+    if (vec) {
+#pragma unroll
+      for (int j = 0; j < NKQ; ++j) {
+        const int e = (tid + 256 * j) * VE, d = e % DP, tt = e / DP;
+        unpack(rk[j], Ks + tt * QS + d, tt < nt);
+        unpack(rq[j], Qs + tt * QS + d, tt < nt);
+      }
+#pragma unroll
+      for (int j = 0; j < NVV; ++j) {
+        const int e = (tid + 256 * j) * VE, c = e % 64, tt = e / 64;
+        unpack(rv[j], Vs + tt * CS + c, tt < nt && col0 + c < V);
+      }
+      if (tb + CL < t_hi) fetch(tb + CL);
+    } else {
+#pragma unroll 8
+      for (int i = tid; i < CL * DP; i += 256) {
+        const int d = i % DP, tt = i / DP;
+        const bool live = tt < nt && d < D;
+        const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+        Ks[tt * QS + d] = live ? act_in(ldf<T>(row, k_off + hd * D + d), act) : 0.f;
+        Qs[tt * QS + d] = live ? act_in(ldf<T>(row, q_off + hd * D + d), act) : 0.f;
+      }
+#pragma unroll 8
+      for (int i = tid; i < CL * 64; i += 256) {
+        const int c = i % 64, tt = i / 64;
+        Vs[tt * CS + c] = (tt < nt && col0 + c < V)
+                              ? act_in(ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col0 + c), act) : 0.f;
+      }
     }
     __syncthreads();
     // ---- P[t][s] = lambda^(t-s) (q_t . k_s) for s <= t; rows of wave w: t = 16 w + ..

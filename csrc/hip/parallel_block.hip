@@ -130,29 +130,31 @@ __global__ void __launch_bounds__(256) relu2_rows_kernel(const T* __restrict__ z
   }
 }
 
-// z[t, e] = x[t, :] . w[e, :] + b[e]: fp32 input rows (a norm's fp32 output), weights in the storage type, fp32 sums. A
-// workgroup takes GT tokens and four weight rows (one a wave), so a weight row is read once per GT tokens.
-template <typename T, int GT>
+// z[t, e] = x[t, :] . w[e, :] + b[e]: fp32 input rows (a norm's fp32 output), weights in the storage type, fp32 sums.
+// For few tokens (decoding; large batches go to the fp32 library product): one wave per (token, weight row). VEC: rows
+// that are multiples of 4 with 8- / 16-byte aligned weights move as vectors, eight loads of a lane in flight.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restrict__ x, const T* __restrict__ w,
-                                                             const T* __restrict__ bias, float* __restrict__ z, int Ttok,
-                                                             int W, int E) {
-  const int t0 = blockIdx.x * GT, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                                                             const T* __restrict__ bias, float* __restrict__ z, int W,
+                                                             int E) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int u = blockIdx.y * 4 + wave;
   if (u >= E) return;
   const T* wr = w + (size_t)u * W;
-  float s[GT];
-#pragma unroll
-  for (int tt = 0; tt < GT; ++tt) s[tt] = 0.f;
-  for (int i = lane; i < W; i += 64) {
-    const float wv = ldf<T>(wr, i);
-#pragma unroll
-    for (int tt = 0; tt < GT; ++tt) s[tt] += x[(size_t)min(t0 + tt, Ttok - 1) * W + i] * wv;
+  const float* xr = x + (size_t)t * W;
+  float s = 0.f;
+  if (VEC) {
+#pragma unroll 8
+    for (int i = 4 * lane; i < W; i += 256) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(xr + i), b = ld4<T>(wr, i);
+      s += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+    }
+  } else {
+#pragma unroll 8
+    for (int i = lane; i < W; i += 64) s += xr[i] * ldf<T>(wr, i);
   }
-#pragma unroll
-  for (int tt = 0; tt < GT; ++tt) {
-    const float tot = wave_sum(s[tt]);
-    if (lane == 0 && t0 + tt < Ttok) z[(size_t)(t0 + tt) * E + u] = tot + (bias ? ldf<T>(bias, u) : 0.f);
-  }
+  s = wave_sum(s);
+  if (lane == 0) z[(size_t)t * E + u] = s + (bias ? ldf<T>(bias, u) : 0.f);
 }
 
 int blocks_for(int64_t total) { return (int)((total + 255) / 256 < 65535 * 8 ? (total + 255) / 256 : 65535 * 8); }
@@ -230,15 +232,16 @@ extern "C" int areal_relu2_rows(const void* z, int64_t row_stride, void* out, in
 extern "C" int areal_router_logits(const float* x, const void* w, const void* bias, float* z, int T, int W, int E, int dt,
                                    hipStream_t st) {
   if (T == 0 || E == 0) return 0;
-#define LAUNCH(TT, GTV)                                                                                              \
-  hipLaunchKernelGGL((router_logits_kernel<TT, GTV>), dim3((T + GTV - 1) / GTV, (E + 3) / 4), dim3(256), 0, st, x,   \
-                     (const TT*)w, (const TT*)bias, z, T, W, E)
+  const bool vec = W % 4 == 0 && ((uintptr_t)w % (dt == 0 ? 8 : 16)) == 0 && ((uintptr_t)x % 16) == 0;
+  const dim3 grid(T, (E + 3) / 4);
+#define LAUNCH(TT, VV)                                                                                            \
+  hipLaunchKernelGGL((router_logits_kernel<TT, VV>), grid, dim3(256), 0, st, x, (const TT*)w, (const TT*)bias, z, W, E)
   if (dt == 0) {
-    if (T < 512) LAUNCH(bf16_t, 1);
-    else LAUNCH(bf16_t, 8);
+    if (vec) LAUNCH(bf16_t, true);
+    else LAUNCH(bf16_t, false);
   } else {
-    if (T < 512) LAUNCH(float, 1);
-    else LAUNCH(float, 8);
+    if (vec) LAUNCH(float, true);
+    else LAUNCH(float, false);
   }
 #undef LAUNCH
   return (int)hipGetLastError();

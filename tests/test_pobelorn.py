@@ -333,7 +333,7 @@ def test_routed_and_shared_experts(device, dtype, W, ff, E, top, shared):
         e["shared"] = {"ff": shared}
         w["shared.gate"], w["shared.up"], w["shared.down"] = sh_in[:shared], sh_in[shared:], mod.shared_down
     w = {k: v.detach().to(F64).cpu() for k, v in w.items()}
-    for T in (1, 9, 70):
+    for T in (1, 9, 70, 300):
         h = torch.randn(T, W, generator=g).to(dtype)
         want = O.moe_ff(h.to(F64), w, e)
         hd = h.to(device)
