@@ -599,8 +599,8 @@ extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, 
                                           int D, int V, float eps, int v_transposed, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (R < 0 || R > D || R % 2 != 0 || n_pos < 1 || (v_first && !lam)) return -1;
-  // few tokens (decoding): a head a wave; many: a token a workgroup
-  const dim3 grid(T, T <= 512 ? (H + G + 3) / 4 : 1);
+  // a head a wave: a token's heads are spread over grid y
+  const dim3 grid(T, (H + G + 3) / 4);
   if (dt == 0)
     hipLaunchKernelGGL(rot_norm_cache_write_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)proj, row_stride,
                        positions, table, n_pos, R, slots, (const bf16_t*)v_first, vf_stride, (const bf16_t*)lam,
