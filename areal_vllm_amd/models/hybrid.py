@@ -476,7 +476,7 @@ class RotaryWindowAttentionMixer(nn.Module):
         heads of 128 on the GPU, otherwise token-major pages of any key and value size."""
         from ..ops.attention import alloc_kv_cache
 
-        self.standard = wattn.standard_layout_ok(self.D, self.V, dtype, device)
+        self.standard = wattn.standard_layout_ok(self.D, self.V, dtype, device) and self.H // self.G <= 16
         if self.standard:
             return alloc_kv_cache(num_pages, self.G, self.D, dtype, device)
         return wattn.alloc_window_cache(num_pages, self.G, self.D, self.V, dtype, device)
@@ -496,7 +496,7 @@ class RotaryWindowAttentionMixer(nn.Module):
             return
         sc = self.rot.get("scaling") or None
         key = ("rot", float(self.rot["base"]), int(self.rot["dims"]), int(n_pos),
-               tuple(sorted((k, float(v)) for k, v in sc.items())) if sc else None)
+               tuple(float(sc[k]) for k in ("factor", "original", "fast", "slow")) if sc else None)
         if key not in tables:
             tables[key] = wattn.rotation_table(float(self.rot["base"]), int(self.rot["dims"]), int(n_pos), device, sc)
         self.table = tables[key]

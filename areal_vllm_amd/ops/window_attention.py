@@ -154,7 +154,8 @@ def rot_norm_cache_write(proj: torch.Tensor, positions: torch.Tensor, table: Opt
 
 def standard_layout_ok(dim: int, vdim: int, dtype, device) -> bool:
     """Whether an attention layer without head mixing, cap, bias or sink can live in the engine's standard cache
-    (K [pages, G, 32, 128], V transposed) and run its matrix-core flash / paged-decode kernels."""
+    (K [pages, G, 32, 128], V transposed) and run its matrix-core flash / paged-decode kernels (which also want at
+    most 16 query heads per key/value head)."""
     return dim == vdim == 128 and dtype == torch.bfloat16 and torch.device(device).type == "cuda"
 
 
