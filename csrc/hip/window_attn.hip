@@ -136,6 +136,86 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_kernel(
   }
 }
 
+// The same for bf16 rows whose head sizes, strides and addresses are multiples of 8 elements (head size <= 512):
+// sixteen lanes a head, every lane 8 consecutive coordinates (four rotation pairs) per 16-byte load, the head's
+// rotated values kept in registers between the sum of squares and the scaling. Values move as 16-byte vectors too.
+template <int NV>
+__global__ void __launch_bounds__(256) rot_norm_cache_write_vec_kernel(
+    const bf16_t* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions,
+    const float* __restrict__ table, int n_pos, int R, const int64_t* __restrict__ slots,
+    const bf16_t* __restrict__ v_first, int64_t vf_stride, const bf16_t* __restrict__ lam_p, bf16_t* __restrict__ q_out,
+    bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache, int H, int G, int D, int V, float eps, int v_transposed) {
+  const int t = blockIdx.x;
+  const bf16_t* row = proj + (size_t)t * row_stride;
+  const int64_t slot = slots[t];
+  const int l16 = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  const size_t page = slot >= 0 ? (size_t)(slot / PAGE) : 0;
+  const int off = slot >= 0 ? (int)(slot % PAGE) : 0;
+  const int pos = min(max(positions[t], 0), n_pos - 1);
+  const float* cs = table + (size_t)pos * R;
+  const int half = R / 2;
+  const int u = blockIdx.y * 16 + grp;
+  if (u < H + G && (u < H || slot >= 0)) {
+    const bf16_t* src = row + (size_t)u * D;
+    bf16_t* dst = u < H ? q_out + ((size_t)t * H + u) * D : kcache + ((page * G + (u - H)) * PAGE + off) * D;
+    float x[NV][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int d0 = 8 * (l16 + 16 * j);
+      if (d0 < D) {
+        const bf16x8 raw = ld8(src + d0);
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const float a = bf2f(raw[e]), b = bf2f(raw[e + 1]);
+          const int pi = (d0 + e) >> 1;
+          if (pi < half) {
+            const float c = cs[pi], sn = cs[half + pi];
+            x[j][e] = a * c - b * sn;
+            x[j][e + 1] = b * c + a * sn;
+          } else {
+            x[j][e] = a;
+            x[j][e + 1] = b;
+          }
+          ss += x[j][e] * x[j][e] + x[j][e + 1] * x[j][e + 1];
+        }
+      }
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float r = 1.f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int d0 = 8 * (l16 + 16 * j);
+      if (d0 < D) {
+        bf16x8 o8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o8[e] = f2bf(x[j][e] * r);
+        st8(dst + d0, o8);
+      }
+    }
+  }
+  if (slot >= 0) {
+    const bf16_t* vsrc = row + (size_t)(H + G) * D;
+    const float lam = v_first ? bf2f(lam_p[0]) : 0.f;
+    for (int i = 8 * (blockIdx.y * 256 + threadIdx.x); i < G * V; i += 8 * 256 * gridDim.y) {
+      const int c = i / V, v = i % V;
+      bf16x8 raw = ld8(vsrc + i);
+      if (v_first) {
+        const bf16x8 f = ld8(v_first + (size_t)t * vf_stride + i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) raw[e] = f2bf((1.f - lam) * bf2f(raw[e]) + lam * bf2f(f[e]));
+      }
+      if (v_transposed) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vcache[((page * G + c) * V + v + e) * PAGE + off] = raw[e];
+      } else {
+        st8(vcache + ((page * G + c) * PAGE + off) * V + v, raw);
+      }
+    }
+  }
+}
+
 struct AttnShape {
   int H, G, D, V, BQ;
   // LDS layout in floats
@@ -599,6 +679,19 @@ extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, 
                                           int D, int V, float eps, int v_transposed, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (R < 0 || R > D || R % 2 != 0 || n_pos < 1 || (v_first && !lam)) return -1;
+  if (dt == 0 && D % 8 == 0 && V % 8 == 0 && D <= 512 && row_stride % 8 == 0 && ((uintptr_t)proj % 16) == 0 &&
+      (!v_first || (vf_stride % 8 == 0 && ((uintptr_t)v_first % 16) == 0))) {
+    const dim3 vgrid(T, (H + G + 15) / 16);
+#define VEC(NVV)                                                                                                    \
+  hipLaunchKernelGGL(rot_norm_cache_write_vec_kernel<NVV>, vgrid, dim3(256), 0, st, (const bf16_t*)proj, row_stride, \
+                     positions, table, n_pos, R, slots, (const bf16_t*)v_first, vf_stride, (const bf16_t*)lam,       \
+                     (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_transposed)
+    if (D <= 128) VEC(1);
+    else if (D <= 256) VEC(2);
+    else VEC(4);
+#undef VEC
+    return (int)hipGetLastError();
+  }
   // a head a wave: a token's heads are spread over grid y
   const dim3 grid(T, (H + G + 3) / 4);
   if (dt == 0)

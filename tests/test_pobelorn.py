@@ -137,12 +137,15 @@ def _slots(pages, lo, hi, device):
 
 @pytest.mark.parametrize("device,dtype", OP_CASES)
 @pytest.mark.parametrize("H,G,D,V,rot", [(4, 2, 16, 8, ROTS[0]), (3, 3, 10, 5, ROTS[2]), (2, 1, 16, 16, ROTS[1]),
-                                         (1, 1, 4, 4, None), (8, 2, 64, 32, ROTS[1])])
+                                         (1, 1, 4, 4, None), (8, 2, 64, 32, ROTS[1]), (8, 8, 128, 128, ROTS[0]),
+                                         (8, 4, 264, 8, ROTS[2])])
 def test_rotation_unit_norm_value_mixing_and_cache_write(device, dtype, H, G, D, V, rot):
     g = torch.Generator().manual_seed(H * 100 + D)
     T, eps, pos0 = 45, 1e-4, 90
-    proj = (torch.randn(T, (H + G) * D + G * V + 7, generator=g) * 2).to(dtype)
-    vf_wide = torch.randn(T, G * V + 3, generator=g).to(dtype)
+    # H = 8: rows, offsets and sizes that are multiples of 8 elements (the kernel's 16-byte form); otherwise odd ones
+    pad, vo = (8, 8) if H == 8 else (7, 2)
+    proj = (torch.randn(T, (H + G) * D + G * V + pad, generator=g) * 2).to(dtype)
+    vf_wide = torch.randn(T, G * V + (16 if H == 8 else 3), generator=g).to(dtype)
     lam = torch.tensor([0.3], dtype=dtype)
     pages = [5, 2, 7, 1, 6]
     slots = _slots(pages, pos0, pos0 + T, device)
@@ -151,7 +154,7 @@ def test_rotation_unit_norm_value_mixing_and_cache_write(device, dtype, H, G, D,
     p64 = proj.to(F64)
     for mixing in (False, True):
         kc, vc = _paged(9, G, D, V, dtype, device)
-        vf = vf_wide.to(device)[:, 2:2 + G * V] if mixing else None
+        vf = vf_wide.to(device)[:, vo:vo + G * V] if mixing else None
         q = wattn.rot_norm_cache_write(proj.to(device), i32(list(range(pos0, pos0 + T)), device), table, slots, kc, vc,
                                        H, eps, vf, lam.to(device) if mixing else None)
         for t in range(T):
@@ -161,7 +164,7 @@ def test_rotation_unit_norm_value_mixing_and_cache_write(device, dtype, H, G, D,
             assert rel_err(q[t].float().cpu(), O.rms(qh, eps)) < tol(dtype)
             v = p64[t, (H + G) * D:(H + G) * D + G * V]
             if mixing:
-                v = (1 - float(lam.to(F64))) * v + float(lam.to(F64)) * vf_wide.to(F64)[t, 2:2 + G * V]
+                v = (1 - float(lam.to(F64))) * v + float(lam.to(F64)) * vf_wide.to(F64)[t, vo:vo + G * V]
             s = int(slots[t])
             if s < 0:
                 continue
