@@ -157,6 +157,42 @@ __global__ void __launch_bounds__(256) router_logits_kernel(const float* __restr
   if (lane == 0) z[(size_t)t * E + u] = s + (bias ? ldf<T>(bias, u) : 0.f);
 }
 
+// bf16 rows whose width, stride and addresses are multiples of 8 elements: 16-byte loads and stores, 8 outputs a thread.
+// GLU = true: act(gate) * up (act 0: SiLU, 1: tanh-GELU); false: max(z, 0)^2.
+template <bool GLU>
+__global__ void __launch_bounds__(256) act_rows_vec_kernel(const bf16_t* __restrict__ in, int64_t row_stride,
+                                                            bf16_t* __restrict__ out, int64_t n, int F, int act) {
+  const int fv = F / 8;
+  const int64_t total = n * fv;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / fv;
+    const int c = 8 * (int)(i % fv);
+    const bf16x8 g = ld8(in + r * row_stride + c);
+    bf16x8 o;
+    if (GLU) {
+      const bf16x8 u = ld8(in + r * row_stride + F + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = bf2f(g[e]);
+        const float a = act == 0 ? x / (1.f + expf(-x))
+                                 : 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+        o[e] = f2bf(a * bf2f(u[e]));
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = fmaxf(bf2f(g[e]), 0.f);
+        o[e] = f2bf(x * x);
+      }
+    }
+    st8(out + r * (int64_t)F + c, o);
+  }
+}
+
+bool rows_vec_ok(const void* in, int64_t row_stride, const void* out, int F, int dt) {
+  return dt == 0 && F % 8 == 0 && row_stride % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0;
+}
+
 int blocks_for(int64_t total) { return (int)((total + 255) / 256 < 65535 * 8 ? (total + 255) / 256 : 65535 * 8); }
 
 }  // namespace
@@ -206,6 +242,11 @@ extern "C" int areal_embed_scale(const int64_t* tokens, const void* embed, float
 extern "C" int areal_glu_rows(const void* gu, int64_t row_stride, void* out, int64_t n, int F, int act, int dt,
                               hipStream_t st) {
   if (n == 0 || F == 0) return 0;
+  if (rows_vec_ok(gu, row_stride, out, F, dt)) {
+    hipLaunchKernelGGL(act_rows_vec_kernel<true>, dim3(blocks_for(n * F / 8)), dim3(256), 0, st, (const bf16_t*)gu,
+                       row_stride, (bf16_t*)out, n, F, act);
+    return (int)hipGetLastError();
+  }
   const int nb = blocks_for(n * F);
   if (dt == 0)
     hipLaunchKernelGGL(glu_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)gu, row_stride, (bf16_t*)out,
@@ -218,6 +259,11 @@ extern "C" int areal_glu_rows(const void* gu, int64_t row_stride, void* out, int
 
 extern "C" int areal_relu2_rows(const void* z, int64_t row_stride, void* out, int64_t n, int F, int dt, hipStream_t st) {
   if (n == 0 || F == 0) return 0;
+  if (rows_vec_ok(z, row_stride, out, F, dt)) {
+    hipLaunchKernelGGL(act_rows_vec_kernel<false>, dim3(blocks_for(n * F / 8)), dim3(256), 0, st, (const bf16_t*)z,
+                       row_stride, (bf16_t*)out, n, F, 0);
+    return (int)hipGetLastError();
+  }
   const int nb = blocks_for(n * F);
   if (dt == 0)
     hipLaunchKernelGGL(relu2_rows_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t*)z, row_stride, (bf16_t*)out,

@@ -97,8 +97,9 @@ def test_embedding_norm_and_closing_sum(device, dtype):
 @pytest.mark.parametrize("device,dtype", OP_CASES)
 def test_activations_on_column_ranges(device, dtype):
     g = torch.Generator().manual_seed(4)
-    for n, Fh, lead in ((7, 24, 5), (1, 3, 0), (33, 130, 16)):
-        wide = (2 * torch.randn(n, lead + 2 * Fh + 3, generator=g)).to(dtype)
+    for n, Fh, lead in ((7, 24, 5), (1, 3, 0), (33, 130, 16), (40, 136, 16), (3, 8, 0)):
+        pad = 8 if (Fh % 8 == 0 and lead % 8 == 0) else 3  # rows of the kernels' 16-byte form, and odd ones
+        wide = (2 * torch.randn(n, lead + 2 * Fh + pad, generator=g)).to(dtype)
         gu = wide.to(device)[:, lead:lead + 2 * Fh]
         a, b = wide[:, lead:lead + Fh].to(F64), wide[:, lead + Fh:lead + 2 * Fh].to(F64)
         out = pb.glu_rows(gu)
