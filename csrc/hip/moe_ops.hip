@@ -477,6 +477,28 @@ __global__ void __launch_bounds__(256) moe_combine_w32_kernel(const T* __restric
     mo_st<T>(out, (size_t)t * H + c, a);
   }
 }
+
+// bf16 rows that are multiples of 8 columns at 16-byte aligned addresses: a thread sums 8 columns from 16-byte loads.
+__global__ void __launch_bounds__(256) moe_combine_w32_vec_kernel(const bf16_t* __restrict__ src,
+                                                                  const int64_t* __restrict__ inv,
+                                                                  const float* __restrict__ w, bf16_t* __restrict__ out,
+                                                                  int k, int H) {
+  const int64_t t = blockIdx.x;
+  const int c = 8 * (blockIdx.y * 256 + threadIdx.x);
+  if (c < H) {
+    float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k; ++j) {
+      const float wj = w[t * k + j];
+      const bf16x8 x = ld8(src + (size_t)inv[t * k + j] * H + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[e] += wj * bf2f(x[e]);
+    }
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = f2bf(a[e]);
+    st8(out + (size_t)t * H + c, o);
+  }
+}
 }  // namespace
 
 extern "C" int areal_clamped_glu(const void* gu, void* out, int64_t n, int F, float limit, float alpha, int dt,
@@ -504,6 +526,11 @@ extern "C" int areal_moe_combine_w32(const void* src, const int64_t* inv, const 
                                      int H, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (k < 1) return -3;
+  if (dt == 0 && H % 8 == 0 && (((uintptr_t)src | (uintptr_t)out) & 15) == 0) {
+    hipLaunchKernelGGL(moe_combine_w32_vec_kernel, dim3((unsigned)T, (H / 8 + 255) / 256), dim3(256), 0, st,
+                       (const bf16_t*)src, inv, w, (bf16_t*)out, k, H);
+    return (int)hipGetLastError();
+  }
   if (dt == 0)
     hipLaunchKernelGGL(moe_combine_w32_kernel<bf16_t>, dim3((unsigned)T, (H + 255) / 256), dim3(256), 0, st, (const bf16_t*)src, inv, w,
                        (bf16_t*)out, k, H);
