@@ -589,6 +589,55 @@ def test_other_sizes_windows_constants_and_orders(device, dtype, which):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes_orders_and_schedules(device, dtype, seed):
+    """Random layer lists (mixer kinds and sizes, windows, kept tokens, rotation constants, with and without
+    feed-forward) fed through random schedules of up to three live requests: portions of 1 .. 100 tokens, requests
+    that skip steps."""
+    import random
+
+    rng = random.Random(seed)
+    for case in range(2):
+        width, vocab, layers = rng.choice([32, 48, 72]), rng.choice([37, 101]), []
+        kv, vdim = rng.choice([1, 2, 3]), rng.choice([8, 20, 32, 64, 128])  # shared by the layers that mix values
+        for _ in range(rng.randint(1, 4)):
+            E = rng.choice([2, 5, 9])
+            mlp = rng.choice(["dense", "moe", "moe", None])
+            if rng.random() < 0.65:
+                dim = rng.choice([8, 12, 64, 128])
+                layers.append(attn(kv * rng.choice([1, 2, 4]), kv, dim, vdim, rng.choice([1, 2, 31, 32, 33, 100, 0]),
+                                   rng.choice([0, 1, 5, 40]), rng.choice([0, 2, dim // 2, dim]), rng.choice([0.1, 0.3]),
+                                   rng.random() < 0.8, rng.choice([100.0, 10000.0]), rng.choice([0, 2.0, 8.0]),
+                                   rng.choice([16, 64]), mlp, rng.choice([8, 20, 64]), E, rng.randint(1, E),
+                                   rng.choice([0, 8, 24])))
+            else:
+                H = rng.choice([1, 2, 3])
+                layers.append(light(H, rng.choice([8, 24, 64, 128]), rng.choice([8, 40, 64, 72]),
+                                    [rng.choice([0.5, 0.9, 0.99, 1.0]) for _ in range(H)], mlp, rng.choice([8, 20, 64]), E,
+                                    rng.randint(1, E), rng.choice([0, 8, 24])))
+        cfg = config(layers, width=width, vocab=vocab, eps=rng.choice([1e-5, 1e-6]), scale=rng.choice([1.0, 7.0]))
+        reqs = {f"q{i}": tokens_of(rng.choice([1, 2, 17, 97, 150]), vocab, 100 * case + i)
+                for i in range(rng.randint(1, 3))}
+        at, steps = {r: 0 for r in reqs}, []
+        while any(at[r] < len(t) for r, t in reqs.items()):
+            step = []
+            for r, t in reqs.items():
+                if at[r] < len(t) and rng.random() > 0.2:
+                    c = min(rng.choice([1, 1, 1, 2, 3, 16, 31, 33, 64, 100]), len(t) - at[r])
+                    step.append((r, t[at[r]:at[r] + c], list(range(c)), at[r] + c == len(t)))
+                    at[r] += c
+            if step:
+                steps.append(step)
+        eng, w = make_engine(cfg, device, dtype, num_pages=24, max_running=3)
+        try:
+            got = replay(eng, steps)
+            for r, t in reqs.items():
+                check_against_oracle(got, t, w, cfg, dtype, r)
+        finally:
+            eng.destroy()
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
 def test_first_tokens_and_long_decoding(device, dtype):
     cfg = config([attn(window=40, keep=2), light(), attn(heads=2, kv=2, window=9, keep=4, mlp=None)])
     eng, w = make_engine(cfg, device, dtype)
