@@ -214,7 +214,8 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     """q [T, H, D] (row b owns tokens cu_q[b]:cu_q[b+1], the LAST positions of its context of ctx_len[b] tokens,
     whose keys / values are in the cache already). mix [H, H] or None. gate [T, H] (a view with unit stride along
     the heads) or None: head h of token t is multiplied by sigmoid(gate[t, h]). `matrix_cores`: bf16 rows of several
-    queries with head sizes 64 / 128 and at most 16 heads run the MFMA kernel (False: always the plain one).
+    queries with head sizes 64 / 128, value sizes 32 / 64 / 128 and at most 16 heads (without `mix`: any number that
+    splits into groups of whole key/value heads) run the MFMA kernel (False: always the plain one).
     Returns [T, H, Dv]."""
     T, H, D = q.shape
     G, V = kcache.shape[1], vcache.shape[3]
