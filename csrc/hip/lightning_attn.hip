@@ -320,6 +320,46 @@ __global__ void __launch_bounds__(256) lightning_out_kernel(const float* __restr
   }
 }
 
+
+// The same for rows that are multiples of 4 at aligned addresses: 16-byte loads of the read-out, 8- / 16-byte loads and
+// stores of gate and result (the weight may sit anywhere in a flat parameter buffer: element loads).
+template <typename T>
+__global__ void __launch_bounds__(256) lightning_out_vec_kernel(const float* __restrict__ obuf, const T* __restrict__ gate,
+                                                                 int64_t gate_stride, const T* __restrict__ w,
+                                                                 T* __restrict__ out, int64_t out_stride, int N,
+                                                                 float eps) {
+  __shared__ float red[16];
+  const size_t t = blockIdx.x;
+  const float* o = obuf + t * (size_t)N;
+  float ss = 0.f;
+  for (int i = 4 * threadIdx.x; i < N; i += 1024) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(o + i);
+    ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)N + eps);
+  for (int i = 4 * threadIdx.x; i < N; i += 1024) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(o + i);
+    float g[4], y[4];
+    if (sizeof(T) == 2) {
+      const bf16x4 gv = *reinterpret_cast<const bf16x4*>(reinterpret_cast<const bf16_t*>(gate) + t * gate_stride + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] = bf2f(gv[e]);
+    } else {
+      const f32x4 gv = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(gate) + t * gate_stride + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] = gv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = v[e] * r * ldf<T>(w, i + e) / (1.f + expf(-g[e]));
+    if (sizeof(T) == 2)
+      *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(out) + t * out_stride + i) =
+          (bf16x4){f2bf(y[0]), f2bf(y[1]), f2bf(y[2]), f2bf(y[3])};
+    else
+      *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(out) + t * out_stride + i) = (f32x4){y[0], y[1], y[2], y[3]};
+  }
+}
+
 }  // namespace
 
 // proj rows hold (at q_off / k_off / v_off) NH query heads of D, NH key heads of D, NH value heads of V; act = 1:
@@ -378,6 +418,17 @@ extern "C" int areal_lightning_scan(const void* proj, int64_t row_stride, int q_
 extern "C" int areal_lightning_out(const float* obuf, const void* gate, int64_t gate_stride, const void* w, void* out,
                                    int64_t out_stride, int T, int N, float eps, int dt, hipStream_t st) {
   if (T == 0) return 0;
+  const uintptr_t al = dt == 0 ? 8 : 16;
+  if (N % 4 == 0 && gate_stride % 4 == 0 && out_stride % 4 == 0 && ((uintptr_t)obuf % 16) == 0 &&
+      ((uintptr_t)gate % al) == 0 && ((uintptr_t)out % al) == 0) {
+    if (dt == 0)
+      hipLaunchKernelGGL(lightning_out_vec_kernel<bf16_t>, dim3(T), dim3(256), 0, st, obuf, (const bf16_t*)gate,
+                         gate_stride, (const bf16_t*)w, (bf16_t*)out, out_stride, N, eps);
+    else
+      hipLaunchKernelGGL(lightning_out_vec_kernel<float>, dim3(T), dim3(256), 0, st, obuf, (const float*)gate,
+                         gate_stride, (const float*)w, (float*)out, out_stride, N, eps);
+    return (int)hipGetLastError();
+  }
   if (dt == 0)
     hipLaunchKernelGGL(lightning_out_kernel<bf16_t>, dim3(T), dim3(256), 0, st, obuf, (const bf16_t*)gate, gate_stride,
                        (const bf16_t*)w, (bf16_t*)out, out_stride, N, eps);
