@@ -870,7 +870,8 @@ class HybridModelRunner(ModelRunner):
         self.hq = self.hkv = 1
         self.sandwich = bool(getattr(self.model, "sandwich", False))
         self.parallel = bool(getattr(self.model, "parallel", False))
-        self.keeps_positions = self.sandwich or self.parallel
+        self.prepost = bool(getattr(self.model, "prepost", False))
+        self.keeps_positions = self.sandwich or self.parallel or self.prepost
         # one cache / state per layer RUN: a layer that runs several times keeps every pass apart
         self.layer_runs = list(getattr(self.model, "layer_runs", range(len(self.model.layers))))
         self.kv, self.state = [], []
@@ -892,6 +893,12 @@ class HybridModelRunner(ModelRunner):
                 H, D, V = blk.mix.state_shape()
                 self.kv.append(None)
                 self.state.append(lightning_ops.alloc_state(self.n_state_slots, H, D, V, self.device))
+            elif blk.kind == "gla":
+                from ..ops import gla as gla_ops
+
+                H, D, V = blk.mix.state_shape()
+                self.kv.append(None)
+                self.state.append(gla_ops.alloc_state(self.n_state_slots, H, D, V, self.device))
             elif blk.kind == "latent_attention":
                 R, P = blk.mix.cache_shape()
                 blk.mix.prepare(self.max_context + 1, tables)
@@ -909,7 +916,7 @@ class HybridModelRunner(ModelRunner):
         self._neg1 = torch.full((1,), -1, dtype=torch.int32, device=self.device)
 
     def _embed(self, ids: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
-        if self.sandwich or self.parallel:  # the fp32 stream starts in `_run_layers`, from the token ids
+        if self.sandwich or self.parallel or self.prepost:  # the fp32 stream starts in `_run_layers`, from the token ids
             return ids
         return self.model.embed_tokens(ids, pos)
 
@@ -933,6 +940,8 @@ class HybridModelRunner(ModelRunner):
             return self._run_layers_sandwich(xc, st)
         if self.parallel:
             return self._run_layers_parallel(xc, st)
+        if self.prepost:
+            return self._run_layers_prepost(xc, st)
         x32 = xc.float() if xc.dtype != torch.float32 else xc.clone()
         alpha, eps = float(cfg.postln_alpha), float(cfg.rms_norm_eps)
         trace = getattr(self, "layer_trace", None)
@@ -991,9 +1000,52 @@ class HybridModelRunner(ModelRunner):
                 trace.append(x32.clone())
         return x32
 
+    def _run_layers_prepost(self, ids: torch.Tensor, st) -> torch.Tensor:
+        """Token ids -> fp32 residual stream after the last layer. Every sublayer is closed by one launch: the norm
+        behind the sublayer, the scaled residual sum, at a layer's end the average over all streams so far (they live
+        in `stack`: X_0 ahead of the first layer, X_(i+1) behind layer i), and the norm the next sublayer reads."""
+        from ..ops import depth_avg as da
+
+        model, cfg = self.model, self.cfg
+        eps, mult = float(cfg.rms_norm_eps), float(cfg.residual_mult)
+        blocks = [model.layers[li] for li in self.layer_runs]
+        T, W = ids.numel(), cfg.hidden_size
+        stack = torch.empty(len(blocks) + 1, T, W, dtype=torch.float32, device=self.device)
+        trace = getattr(self, "layer_trace", None)
+        h32, hc = da.embed_pos_norm(ids, st.positions, model.embed, model.pos, blocks[0].norm1, eps, self.dtype,
+                                    stack[0], want32=False)
+        x = stack[0]
+        for ri, blk in enumerate(blocks):
+            cache = self.state[ri] if blk.kind == "gla" else self.kv[ri]
+            y = blk.mix.step(hc, st, cache)
+            nxt = blocks[ri + 1].norm1 if ri + 1 < len(blocks) else None
+            nst = ri + 2 if blk.dwa is not None else 0
+            if blk.mlp is not None:
+                # the layer's stream in progress lives in its slot of the stack: X_ri itself stays what it was
+                x, h32, hc = da.norm_add_avg_norm(x, y, blk.norm1b, mult, None, 0, None, blk.norm2, eps, self.dtype,
+                                                  want32=blk.needs32, out=stack[ri + 1])
+                y = blk.mlp(None, hc, h32)
+                x, h32, hc = da.norm_add_avg_norm(x, y, blk.norm2b, mult, stack if nst else None, nst, blk.dwa, nxt,
+                                                  eps, self.dtype, out=stack[ri + 1])
+            else:
+                x, h32, hc = da.norm_add_avg_norm(x, y, blk.norm1b, mult, stack if nst else None, nst, blk.dwa, nxt,
+                                                  eps, self.dtype, out=stack[ri + 1])
+            if trace is not None:
+                trace.append(x.clone())
+        return x
+
     def _final_logits(self, h, residual, fp32: bool = False) -> torch.Tensor:
         from ..ops.post_norm import scaled_add_norm
 
+        if self.prepost:
+            from ..ops import depth_avg as da
+
+            want32 = fp32 or self.keep_logits
+            _, x32, xc = da.norm_add_avg_norm(h.contiguous(), None, None, 1.0, None, 0, None, self.model.norm,
+                                              float(self.cfg.rms_norm_eps), self.dtype, want32=want32)
+            if want32:
+                return F.linear(x32, self.model.head_weight.float())
+            return F.linear(xc, self.model.head_weight)
         if self.parallel:
             from ..ops import parallel_block as pb
 
@@ -1038,6 +1090,15 @@ class HybridModelRunner(ModelRunner):
 
         nsplit, ws = 1, None
         latent = [blk.mix for blk in self.model.layers if blk.kind == "latent_attention"]
+        if self.prepost and self.device.type == "cuda":
+            # mixers of several kinds share one workspace; each takes its own share of the step's splits
+            need = [(m.decode_splits(Bp, self.max_context), m.H * (m.R if blk.kind == "latent_attention" else m.V), m.H)
+                    for blk in self.model.layers if blk.kind != "gla" for m in (blk.mix,)]
+            nsplit = max([n for n, _, _ in need] or [1])
+            if nsplit > 1:
+                ws = (torch.empty(Bp * max(n * a for n, a, _ in need), dtype=torch.float32, device=self.device),
+                      torch.empty(Bp * max(n * h for n, _, h in need) * 2, dtype=torch.float32, device=self.device))
+            return nsplit, ws
         if latent and self.device.type == "cuda":
             from ..ops import latent_attention as lattn
 

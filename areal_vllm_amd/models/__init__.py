@@ -4,7 +4,8 @@ from .transformer import FlatParams, Transformer  # noqa: F401
 from .hybrid import HybridConfig, HybridDecoder  # noqa: F401
 
 # model family (``ModelConfig.family``) -> class; every family not listed is a ``Transformer`` variant
-MODEL_CLASSES = {"kuzanex": HybridDecoder, "lufivik": HybridDecoder, "pobelorn": HybridDecoder}
+MODEL_CLASSES = {"kuzanex": HybridDecoder, "lufivik": HybridDecoder, "pobelorn": HybridDecoder,
+                 "zusotar": HybridDecoder}
 
 
 def model_class(cfg: ModelConfig):

@@ -13,7 +13,8 @@ from typing import Any, Dict, List, Optional
 
 
 # config.json "architecture" -> reader in models/hybrid.py (designs given as a list of layers)
-LAYER_LIST_DESIGNS = {"Kuzanex": "kuzanex_config", "Lufivik": "lufivik_config", "Pobelorn": "pobelorn_config"}
+LAYER_LIST_DESIGNS = {"Kuzanex": "kuzanex_config", "Lufivik": "lufivik_config", "Pobelorn": "pobelorn_config",
+                      "Zusotar": "zusotar_config"}
 
 
 @dataclasses.dataclass

@@ -23,11 +23,24 @@ ff:         squared-ReLU MLP, or routed gated experts (router with bias, softmax
             shared expert
 Embedding:  table row times a constant; the logits come from the same table
 
+The Zusotar design is the fourth member. Its sublayers sit between two RMS norms (weights stored around zero):
+
+Layer:      x <- x + m norm1b(mixer(norm1(x)));  x <- x + m norm2b(ff(norm2(x)));  then a learned average over depth:
+            what goes on is sum_j a[j] X_j over the stream ahead of the first layer and behind every layer so far
+Mixers:     causal attention through a shared latent (queries straight from the input, rotated neighbour pairs, one sink
+            logit per head in the softmax denominator);  grouped-query window attention without rotation whose values
+            have unit RMS, with a learned logarithmic distance penalty and an element-wise sigmoid gate;  gated linear
+            attention (a decay per key channel from a low-rank projection, fp32 state)
+ff:         gated MLP, or routed gated experts chosen by sigmoid scores among the best groups of experts, weighted by
+            the scores as they are, plus a shared expert
+Embedding:  table row plus a learned vector per position
+
 The mechanisms are separate modules with their constants as constructor arguments (``WindowAttentionMixer``,
 ``MLSTMMixer``, ``XieluMLP``, ``LatentAttentionMixer``, ``RoutedGLUExperts``, ``RotaryWindowAttentionMixer``,
-``LightningMixer``, ``SquaredReluMLP``, ``RoutedSwiGLUExperts``); what they compute is documented with
+``LightningMixer``, ``SquaredReluMLP``, ``RoutedSwiGLUExperts``, ``LogBiasWindowAttentionMixer``, ``GLAMixer``,
+``GatedMLP``); what they compute is documented with
 their kernels (``ops/window_attention.py``, ``ops/mlstm.py``, ``ops/post_norm.py``, ``ops/latent_attention.py``,
-``ops/sandwich.py``, ``ops/lightning.py``, ``ops/parallel_block.py``). The modules hold parameters and know how to run ONE step on the tensors of a
+``ops/sandwich.py``, ``ops/lightning.py``, ``ops/parallel_block.py``, ``ops/gla.py``, ``ops/depth_avg.py``). The modules hold parameters and know how to run ONE step on the tensors of a
 batch plan; paged caches, state slots and the loop over layers belong to the model runner
 (``inference/model_runner.py::HybridModelRunner``).
 """
@@ -41,6 +54,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
+from ..ops import depth_avg as davg
+from ..ops import gla as gla_ops
 from ..ops import lightning as lightning_ops
 from ..ops import mlstm as mlstm_ops
 from ..ops import parallel_block as pblock
@@ -59,9 +74,12 @@ class HybridConfig(ModelConfig):
     layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
     postln_alpha: float = 1.0
     design: str = "Kuzanex"
-    # "post_norm": norm after every sum; "sandwich": norms before and after a sublayer; "parallel": one norm, mixer and
-    # feed-forward read it and are added together
+    # "post_norm": norm after every sum; "sandwich": layer norms before and after a sublayer, gated; "parallel": one
+    # norm, mixer and feed-forward read it and are added together; "prepost": RMS norms before and after a sublayer,
+    # the normed output times `residual_mult` added to the stream, optionally averaged over depth
     block_style: str = "post_norm"
+    residual_mult: float = 1.0  # factor on every normed sublayer output ("prepost" designs)
+    depth_average: bool = False  # the stream that leaves a layer is a learned average of all streams so far
     embed_scale: float = 1.0  # factor on the embedding rows ("parallel" designs)
     loop: Optional[Dict[str, int]] = None  # layers start .. stop - 1 run `times` times in a row
     canon_taps: int = 0  # taps of the causal convolution on a mixer's input (0: none)
@@ -69,7 +87,7 @@ class HybridConfig(ModelConfig):
 
     @property
     def has_recurrent_state(self) -> bool:
-        return (any(l["type"] in ("mlstm", "lightning") for l in self.layers) or self.canon_taps > 1
+        return (any(l["type"] in ("mlstm", "lightning", "gla") for l in self.layers) or self.canon_taps > 1
                 or self.bigram is not None)
 
     @property
@@ -86,6 +104,8 @@ class HybridConfig(ModelConfig):
             return self._n_params_sandwich(with_embedding)
         if self.block_style == "parallel":
             return self._n_params_parallel(with_embedding)
+        if self.block_style == "prepost":
+            return self._n_params_prepost(with_embedding)
         W, n = self.hidden_size, 1
         for l in self.layers:
             m = l["mixer"]
@@ -136,7 +156,41 @@ class HybridConfig(ModelConfig):
                     n += 3 * W * e["shared"]["ff"]
         return n + (self.vocab_size * W if with_embedding else 0)
 
+    def _n_params_prepost(self, with_embedding: bool) -> int:
+        W = self.hidden_size
+        n = W  # final norm
+        for i, l in enumerate(self.layers):
+            m = l["mixer"]
+            H, D, V = m["heads"], m["dim"], m["vdim"]
+            if l["type"] == "attention":
+                G = m["kv_heads"]
+                n += W * (H * D + G * D + G * V + H * V) + 2 * H + W * H * V
+            elif l["type"] == "latent_attention":
+                P, R = m["rot_dim"], m["kv_rank"]
+                n += W * (H * (D + P) + R + P) + R + R * H * (D + V) + H + W * H * V
+            else:
+                r = m["decay_rank"]
+                n += W * (2 * H * D + 2 * H * V + r) + r * H * D + H * D + V + W * H * V
+            n += 2 * W + (i + 2 if self.depth_average else 0)
+            e = l.get("mlp")
+            if e:
+                n += 2 * W
+                if e["kind"] == "dense":
+                    n += 3 * W * e["ff"]
+                else:
+                    n += e["router"]["experts"] * (W + 3 * W * e["expert"]["ff"])
+                    if e.get("shared"):
+                        n += 3 * W * e["shared"]["ff"]
+        if with_embedding:
+            n += 2 * self.vocab_size * W + (self.max_position_embeddings * W if self.pos_embed == "learned" else 0)
+        return n
+
     def to_hf_dict(self) -> Dict[str, Any]:
+        if self.block_style == "prepost":
+            layers = json.loads(json.dumps(self.layers))  # gla entries carry `decay_rank` (a checkpoint's shapes give it too)
+            return {"architecture": self.design, "layers": layers, "max_positions": self.max_position_embeddings,
+                    "norm": {"eps": self.rms_norm_eps}, "residual_mult": self.residual_mult,
+                    "vocab": self.vocab_size, "width": self.hidden_size}
         if self.block_style == "parallel":
             return {"architecture": self.design, "embedding": {"scale": self.embed_scale},
                     "layers": json.loads(json.dumps(self.layers)), "norm": {"eps": self.rms_norm_eps},
@@ -271,6 +325,64 @@ def pobelorn_config_from_dir(path: str) -> HybridConfig:
         return pobelorn_config(json.load(f))
 
 
+def zusotar_config(d: Dict[str, Any], decay_ranks: Optional[Dict[int, int]] = None) -> HybridConfig:
+    """config.json of a Zusotar checkpoint -> HybridConfig. Every size and constant is taken from it; the rank of a gla
+    layer's decay projection is a tensor's shape (`decay_ranks`: layer index -> rank, or `decay_rank` in the layer's
+    mixer entry)."""
+    layers = []
+    for i, l in enumerate(d["layers"]):
+        if l["type"] not in ("attention", "latent_attention", "gla"):
+            raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        mlp = l.get("mlp")
+        if mlp is not None and mlp.get("kind") not in ("dense", "moe"):
+            raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+        m = json.loads(json.dumps(l["mixer"]))
+        if l["type"] == "attention":
+            if int(m["heads"]) % int(m.get("kv_heads", m["heads"])):
+                raise ValueError(f"layer {i}: heads is not a multiple of kv_heads")
+        elif l["type"] == "latent_attention":
+            if int(m["rot"]["dims"]) != int(m["rot_dim"]) or int(m["rot_dim"]) % 2:
+                raise ValueError(f"layer {i}: the rotary part has rot_dim (an even number of) dimensions")
+        else:
+            if decay_ranks and i in decay_ranks:
+                m["decay_rank"] = int(decay_ranks[i])
+            if "decay_rank" not in m:
+                raise ValueError(f"layer {i}: the rank of the decay projection is not known")
+        if mlp is not None and mlp["kind"] == "moe":
+            g = mlp["router"].get("groups")
+            if g and (int(mlp["router"]["experts"]) % int(g["count"]) or not 1 <= int(g["keep"]) <= int(g["count"])):
+                raise ValueError(f"layer {i}: the expert groups do not fit the experts")
+        layers.append({"type": l["type"], "mixer": m, "mlp": json.loads(json.dumps(mlp)) if mlp is not None else None})
+    att = next((l["mixer"] for l in layers), None)
+    widths = [(e["ff"] if e["kind"] == "dense" else e["expert"]["ff"]) for e in (l["mlp"] for l in layers) if e]
+    return HybridConfig(
+        family="zusotar", design="Zusotar", block_style="prepost", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), n_layers=len(layers), n_q_heads=int(att["heads"]) if att else 1,
+        n_kv_heads=int(att.get("kv_heads", 1)) if att else 1, head_dim=int(att["dim"]) if att else 1,
+        intermediate_size=max(widths or [0]), rms_norm_eps=float(d["norm"]["eps"]),
+        max_position_embeddings=int(d["max_positions"]), tie_word_embeddings=False, qkv_bias=False,
+        pos_embed="learned", layers=layers, residual_mult=float(d.get("residual_mult", 1.0)), depth_average=True,
+        eos_token_id=d.get("eos_token_id"), pad_token_id=d.get("pad_token_id"))
+
+
+def zusotar_config_from_dir(path: str) -> HybridConfig:
+    """config.json plus one look at the checkpoint's tensor shapes (the rank of every decay projection)."""
+    with open(os.path.join(path, "config.json")) as f:
+        d = json.load(f)
+    ranks: Dict[int, int] = {}
+    want = {f"l{i}.mix.a1": i for i, l in enumerate(d["layers"]) if l["type"] == "gla"}
+    if want:
+        from safetensors import safe_open
+
+        for fn in sorted(os.listdir(path)):
+            if fn.endswith(".safetensors"):
+                with safe_open(os.path.join(path, fn), framework="pt") as f:
+                    for name in f.keys():
+                        if name in want:
+                            ranks[want[name]] = int(f.get_slice(name).get_shape()[0])
+    return zusotar_config(d, ranks)
+
+
 class StepTensors:
     """What one batch plan hands to the mixers (all on the device): rows of the packed token batch (`cu_q`, longest
     row `max_q`), each row's context length after the step, cache slot of every token, page tables, position of each
@@ -374,14 +486,25 @@ class LatentAttentionMixer(nn.Module):
     latents are scored directly) and the attended latents are expanded to values afterwards."""
 
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int,
-                 scale: float, window: int, rot_base: float, eps: float, dtype, device):
+                 scale: float, window: int, rot_base: float, eps: float, dtype, device, head_gate: bool = True,
+                 sink: bool = False, neighbour_pairs: bool = False):
+        """`q_rank` = 0: the queries come straight out of the input projection (no query latent, no norm of it).
+        `head_gate`: one sigmoid gate per head from the same projection. `sink`: one learned logit per head in the
+        softmax denominator. `neighbour_pairs`: rotation pairs are columns (2i, 2i + 1) instead of (i, i + P/2)."""
         super().__init__()
         self.H, self.D, self.P, self.V, self.Q, self.R = heads, dim, rot_dim, vdim, q_rank, kv_rank
         self.scale, self.window, self.rot_base, self.eps = float(scale), int(window), float(rot_base), float(eps)
-        self.proj = nn.Parameter(torch.empty(q_rank + kv_rank + rot_dim + heads, width, dtype=dtype, device=device))
-        self.q_norm = nn.Parameter(torch.ones(q_rank, dtype=dtype, device=device))
+        self.head_gate, self.neighbour_pairs = bool(head_gate), bool(neighbour_pairs)
+        self.n_q = q_rank if q_rank > 0 else heads * (dim + rot_dim)  # leading columns of the projection
+        self.proj = nn.Parameter(torch.empty(self.n_q + kv_rank + rot_dim + (heads if head_gate else 0), width,
+                                             dtype=dtype, device=device))
         self.c_norm = nn.Parameter(torch.ones(kv_rank, dtype=dtype, device=device))
-        self.uq = nn.Parameter(torch.empty(heads * (dim + rot_dim), q_rank, dtype=dtype, device=device))
+        self.sink = nn.Parameter(torch.zeros(heads, dtype=dtype, device=device)) if sink else None
+        if q_rank > 0:
+            self.q_norm = nn.Parameter(torch.ones(q_rank, dtype=dtype, device=device))
+            self.uq = nn.Parameter(torch.empty(heads * (dim + rot_dim), q_rank, dtype=dtype, device=device))
+        else:
+            self.q_norm = self.uq = None
         self.uk = nn.Parameter(torch.empty(heads * dim, kv_rank, dtype=dtype, device=device))
         self.uv = nn.Parameter(torch.empty(heads * vdim, kv_rank, dtype=dtype, device=device))
         self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype, device=device))
@@ -397,18 +520,31 @@ class LatentAttentionMixer(nn.Module):
             tables[key] = lattn.rotary_table(self.rot_base, self.P, int(n_pos), self.proj.device)
         self.table = tables[key]
 
+    def decode_splits(self, batch: int, max_context: int) -> int:
+        return lattn.decode_splits(batch, self.window, max_context, self.H)
+
     def step(self, hc: torch.Tensor, st: StepTensors, cache: torch.Tensor) -> torch.Tensor:
         T = hc.shape[0]
-        H, D, P, V, Q, R = self.H, self.D, self.P, self.V, self.Q, self.R
+        H, D, P, V, Q, R, nq = self.H, self.D, self.P, self.V, self.Q, self.R, self.n_q
         proj = F.linear(hc, self.proj)
-        cq = lattn.latent_prep(proj, Q, R, P, self.q_norm, self.c_norm, st.positions, st.slots, cache, self.table,
-                               self.eps)
-        q = F.linear(cq, self.uq).view(T, H, D + P)
+        if Q > 0:
+            cq = lattn.latent_prep(proj, Q, R, P, self.q_norm, self.c_norm, st.positions, st.slots, cache, self.table,
+                                   self.eps, self.neighbour_pairs)
+            q = F.linear(cq, self.uq).view(T, H, D + P)
+        else:  # the queries are the projection's leading columns, read in place
+            lattn.latent_prep(proj[:, nq:], 0, R, P, None, self.c_norm, st.positions, st.slots, cache, self.table,
+                              self.eps, self.neighbour_pairs)
+            q = proj[:, :nq].view(T, H, D + P)
+        nsplit = 1
+        if st.max_q == 1 and st.nsplit > 1:  # this mixer's own share of the step's key-range splits
+            nsplit = min(st.nsplit, self.decode_splits(T, self.table.shape[0] - 1))
         # q~_h = W_uk[h]^T q^n_h: one batched product over the heads
         q_lat = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk.view(H, D, R)).transpose(0, 1).contiguous()
         o_lat = lattn.latent_attention(q, q_lat, cache, st.block_tables, st.cu_q, st.ctx_len, st.max_q, D, P,
-                                       self.scale, self.window, self.table, gate=proj[:, Q + R + P:],
-                                       nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace)
+                                       self.scale, self.window, self.table,
+                                       gate=proj[:, nq + R + P:] if self.head_gate else None,
+                                       nsplit=nsplit, workspace=st.workspace, neighbours=self.neighbour_pairs,
+                                       sink=self.sink)
         o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, V, R).transpose(1, 2)).transpose(0, 1)
         return F.linear(o.reshape(T, H * V), self.o)
 
@@ -573,12 +709,23 @@ class RoutedSwiGLUExperts(nn.Module):
     on the device). A shared expert of the same form (`shared_ff` > 0) runs for every token and is added; its
     gate | up rows are part of the block's in-projection."""
 
-    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int, dtype, device):
+    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int, dtype, device,
+                 scoring: str = "softmax_chosen", groups=None, router_bias: bool = True, own_shared_in: bool = False):
+        """`scoring` = "softmax_chosen": as above. "sigmoid": the scores are sigmoid(logits), the `top` largest are
+        chosen and are the weights as they are; with `groups` = (count, keep) the experts form `count` equal groups of
+        neighbours, a group scores the sum of its two largest scores and only members of the `keep` best groups can
+        be chosen. `own_shared_in`: the shared expert's gate | up rows are a parameter of this module (for blocks
+        that have no common in-projection)."""
         super().__init__()
-        assert 1 <= top <= experts
+        assert 1 <= top <= experts and scoring in ("softmax_chosen", "sigmoid")
         self.E, self.k, self.ff, self.shared_ff = experts, top, ff, int(shared_ff)
+        self.scoring = scoring
+        self.groups = (int(groups[0]), int(groups[1])) if groups else (1, 1)
+        assert experts % self.groups[0] == 0 and 1 <= self.groups[1] <= self.groups[0]
         self.router = nn.Parameter(torch.empty(experts, width, dtype=dtype, device=device))
-        self.router_bias = nn.Parameter(torch.zeros(experts, dtype=dtype, device=device))
+        self.router_bias = nn.Parameter(torch.zeros(experts, dtype=dtype, device=device)) if router_bias else None
+        self.shared_in = (nn.Parameter(torch.empty(2 * shared_ff, width, dtype=dtype, device=device))
+                          if own_shared_in and shared_ff > 0 else None)
         self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width, dtype=dtype, device=device))
         self.down = nn.Parameter(torch.empty(experts, width, ff, dtype=dtype, device=device))
         self.shared_down = (nn.Parameter(torch.empty(width, shared_ff, dtype=dtype, device=device))
@@ -590,15 +737,194 @@ class RoutedSwiGLUExperts(nn.Module):
     def forward(self, cols: torch.Tensor, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
         # fp32 products on the norm's fp32 output when there is one, else on its rounding
         z = pblock.router_logits(h32 if h32 is not None else hc.float(), self.router, self.router_bias)
-        # softmax over all logits, the k largest re-normalised: the softmax over the chosen logits
-        topv, topi = moe_ops.moe_topk(z, self.k, True, out_dtype=torch.float32)
+        if self.scoring == "sigmoid":
+            topv, topi = moe_ops.moe_group_topk(z, self.k, self.groups[0], self.groups[1])
+        else:  # softmax over all logits, the k largest re-normalised: the softmax over the chosen logits
+            topv, topi = moe_ops.moe_topk(z, self.k, True, out_dtype=torch.float32)
         order, inv, src_row, offsets = moe_ops.moe_sort(topi.reshape(-1), self.E, self.k)
         xs = moe_ops._gather_rows(hc, src_row)
         a = pblock.glu_rows(grouped_gemm_rows(xs, self.gate_up, offsets))
         y = moe_ops.combine_rows_w32(grouped_gemm_rows(a, self.down, offsets), inv, topv)
         if self.shared_down is not None:
+            if self.shared_in is not None:
+                cols = F.linear(hc, self.shared_in)
             y = torch.addmm(y, pblock.glu_rows(cols), self.shared_down.t())
         return y
+
+
+class LogBiasWindowAttentionMixer(nn.Module):
+    """Grouped-query attention without rotation (``ops/window_attention.py``): q | k | v | gate come out of ONE
+    projection; every value head is divided by its root mean square (no weight) and cached so; the score is
+    q . k * scale - r1_h ln(1 + r2_h (i - j)) with two learned numbers per head; sliding window; ordinary softmax; the
+    heads' outputs are multiplied element by element with sigmoid(gate) ahead of the output projection."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, window: int,
+                 v_norm: bool, eps: float, dtype, device):
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.H, self.G, self.D, self.V, self.eps, self.v_norm = heads, kv_heads, dim, vdim, float(eps), bool(v_norm)
+        self.shape = wattn.ScoreShape(scale=float(scale), window=int(window))
+        self.n_qkv = (heads + kv_heads) * dim + kv_heads * vdim
+        self.proj = nn.Parameter(torch.empty(self.n_qkv + heads * vdim, width, dtype=dtype, device=device))
+        self.r1 = nn.Parameter(torch.zeros(heads, dtype=dtype, device=device))
+        self.r2 = nn.Parameter(torch.zeros(heads, dtype=dtype, device=device))
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype, device=device))
+        self.max_context = 1 << 30
+
+    def cache_shape(self):
+        return self.G, self.D, self.V
+
+    def prepare(self, n_pos: int, tables: Dict[Any, torch.Tensor], device):
+        self.max_context = int(n_pos) - 1
+
+    def decode_splits(self, batch: int, max_context: int) -> int:
+        return wattn.decode_splits(batch, self.shape.window, max_context)
+
+    def step(self, hc: torch.Tensor, st: StepTensors, cache) -> torch.Tensor:
+        kc, vc = cache
+        T = hc.shape[0]
+        proj = F.linear(hc, self.proj)
+        q = wattn.qkv_vnorm_cache_write(proj, st.slots, kc, vc, self.H, self.eps, self.v_norm)
+        nsplit = 1
+        if st.max_q == 1 and st.nsplit > 1:
+            nsplit = min(st.nsplit, self.decode_splits(T, self.max_context))
+        o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
+                                   nsplit=nsplit, workspace=st.workspace, gate=proj[:, self.n_qkv:],
+                                   log_bias=(self.r1, self.r2))
+        return F.linear(o.view(T, self.H * self.V), self.o)
+
+
+class GLAMixer(nn.Module):
+    """Gated linear attention (``ops/gla.py``): q | k | v | output gate | the low-rank input of the decay logits come
+    out of ONE projection; the decay logits are the low-rank product plus a bias, formed in fp32; per key channel the
+    state decays by sigmoid(logit)^(1 / tau); per-head RMS norm (one weight vector shared by the heads) and a SiLU
+    gate on the read-out."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, tau: float, decay_rank: int, q_scale: float,
+                 eps: float, dtype, device):
+        super().__init__()
+        self.H, self.D, self.V, self.rank = heads, dim, vdim, int(decay_rank)
+        self.tau, self.q_scale, self.eps = float(tau), float(q_scale), float(eps)
+        self.n_main = 2 * heads * dim + 2 * heads * vdim
+        self.proj = nn.Parameter(torch.empty(self.n_main + self.rank, width, dtype=dtype, device=device))
+        self.a2 = nn.Parameter(torch.empty(heads * dim, self.rank, dtype=dtype, device=device))
+        self.a2_bias = nn.Parameter(torch.zeros(heads * dim, dtype=dtype, device=device))
+        self.norm = nn.Parameter(torch.ones(vdim, dtype=dtype, device=device))
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype, device=device))
+
+    def state_shape(self):
+        return self.H, self.D, self.V
+
+    def step(self, hc: torch.Tensor, st: StepTensors, state: torch.Tensor) -> torch.Tensor:
+        H, D, V = self.H, self.D, self.V
+        proj = F.linear(hc, self.proj)
+        low = proj[:, self.n_main:]
+        if low.dtype == torch.float32:
+            z = F.linear(low, self.a2)
+        elif low.is_cuda:  # 16-bit operands, fp32 accumulation AND fp32 logits
+            z = torch.mm(low, self.a2.t(), out_dtype=torch.float32)
+        else:
+            z = F.linear(low.float(), self.a2.float())
+        o = gla_ops.gla_scan(proj, 0, H * D, 2 * H * D, z, self.a2_bias, self.tau, self.q_scale, st.cu_q, st.first_pos,
+                             st.state_slots, state, max_q=st.max_q)
+        y = gla_ops.gla_out(o, proj[:, 2 * H * D + H * V:self.n_main], self.norm, self.eps)
+        return F.linear(y, self.o)
+
+
+class GatedMLP(nn.Module):
+    """down(act(gate h) * (up h)); gate | up are one projection."""
+
+    def __init__(self, width: int, ff: int, act: str, dtype, device):
+        super().__init__()
+        self.ff, self.act = ff, act
+        self.gate_up = nn.Parameter(torch.empty(2 * ff, width, dtype=dtype, device=device))
+        self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype, device=device))
+
+    def forward(self, cols, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
+        return F.linear(pblock.glu_rows(F.linear(hc, self.gate_up), self.act), self.down)
+
+
+class PrePostBlock(nn.Module):
+    """A layer whose sublayers sit between two RMS norms: x <- x + mult * norm_b(sublayer(norm(x))), for the mixer and
+    (when the layer has one) the feed-forward; the norms' weights are stored around zero. With `depth_average` the
+    layer owns the weights of the average over all streams so far (`n_streams` of them, its own result last). The
+    runner closes every sublayer with one launch that also forms the norm the next sublayer reads."""
+
+    def __init__(self, cfg: HybridConfig, spec: Dict[str, Any], n_streams: int, dtype, device):
+        super().__init__()
+        W, m, eps = cfg.hidden_size, spec["mixer"], cfg.rms_norm_eps
+        self.kind = spec["type"]
+        if self.kind == "attention":
+            self.mix = LogBiasWindowAttentionMixer(
+                W, int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m.get("scale", float(m["dim"]) ** -0.5)), int((m.get("mask") or {}).get("size") or 0), True, eps,
+                dtype, device)
+        elif self.kind == "latent_attention":
+            self.mix = LatentAttentionMixer(
+                W, int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), 0, int(m["kv_rank"]),
+                float(m.get("scale", (int(m["dim"]) + int(m["rot_dim"])) ** -0.5)),
+                int((m.get("mask") or {}).get("size") or 0), float(m["rot"]["base"]), eps, dtype, device,
+                head_gate=False, sink=True, neighbour_pairs=True)
+        else:
+            self.mix = GLAMixer(W, int(m["heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])), float(m["tau"]),
+                                int(m["decay_rank"]), float(m["dim"]) ** -0.5, eps, dtype, device)
+
+        def vec():
+            return nn.Parameter(torch.zeros(W, dtype=dtype, device=device))
+
+        self.norm1, self.norm1b = vec(), vec()
+        e = spec.get("mlp")
+        self.mlp = None
+        if e:
+            self.norm2, self.norm2b = vec(), vec()
+            if e["kind"] == "dense":
+                self.mlp = GatedMLP(W, int(e["ff"]), "silu", dtype, device)
+            else:
+                g = e["router"].get("groups")
+                self.mlp = RoutedSwiGLUExperts(
+                    W, int(e["expert"]["ff"]), int(e["router"]["experts"]), int(e["router"]["top"]),
+                    int((e.get("shared") or {}).get("ff", 0)), dtype, device, scoring="sigmoid",
+                    groups=(int(g["count"]), int(g["keep"])) if g else None, router_bias=False, own_shared_in=True)
+        self.needs32 = isinstance(self.mlp, RoutedSwiGLUExperts)  # the router reads the norm's fp32 output
+        self.dwa = (nn.Parameter(torch.zeros(n_streams, dtype=dtype, device=device)) if cfg.depth_average else None)
+
+    def state_shape(self):
+        return None
+
+    def checkpoint_tensors(self, p: str) -> Dict[str, torch.Tensor]:
+        m = self.mix
+        out = {p + "norm1": self.norm1.data, p + "norm1b": self.norm1b.data, p + "mix.o": m.o.data}
+        if self.dwa is not None:
+            out[p + "dwa"] = self.dwa.data
+        w = m.proj.data
+        if self.kind == "attention":
+            a, b = m.H * m.D, (m.H + m.G) * m.D
+            out.update({p + "mix.q": w[:a], p + "mix.k": w[a:b], p + "mix.v": w[b:m.n_qkv], p + "mix.g": w[m.n_qkv:],
+                        p + "mix.r1": m.r1.data, p + "mix.r2": m.r2.data})
+        elif self.kind == "latent_attention":
+            out.update({p + "mix.q": w[:m.n_q], p + "mix.dkv": w[m.n_q:], p + "mix.dkv.norm": m.c_norm.data,
+                        p + "mix.uk": m.uk.data, p + "mix.uv": m.uv.data, p + "mix.sink": m.sink.data})
+        else:
+            a, b, c = m.H * m.D, 2 * m.H * m.D, 2 * m.H * m.D + m.H * m.V
+            out.update({p + "mix.q": w[:a], p + "mix.k": w[a:b], p + "mix.v": w[b:c], p + "mix.g": w[c:m.n_main],
+                        p + "mix.a1": w[m.n_main:], p + "mix.a2": m.a2.data, p + "mix.a2.b": m.a2_bias.data,
+                        p + "mix.norm": m.norm.data})
+        e, q = self.mlp, p + "mlp."
+        if e is not None:
+            out[p + "norm2"], out[p + "norm2b"] = self.norm2.data, self.norm2b.data
+        if isinstance(e, GatedMLP):
+            out[q + "gate"], out[q + "up"], out[q + "down"] = e.gate_up.data[:e.ff], e.gate_up.data[e.ff:], e.down.data
+        elif e is not None:
+            out[q + "router"] = e.router.data
+            for i in range(e.E):
+                out[q + f"e{i}.gate"] = e.gate_up.data[i, :e.ff]
+                out[q + f"e{i}.up"] = e.gate_up.data[i, e.ff:]
+                out[q + f"e{i}.down"] = e.down.data[i]
+            if e.shared_down is not None:
+                sf = e.shared_ff
+                out[q + "shared.gate"], out[q + "shared.up"] = e.shared_in.data[:sf], e.shared_in.data[sf:]
+                out[q + "shared.down"] = e.shared_down.data
+        return out
 
 
 class ParallelBlock(nn.Module):
@@ -794,8 +1120,18 @@ class HybridDecoder(nn.Module):
         self.embed = nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device))
         self.sandwich = cfg.block_style == "sandwich"
         self.parallel = cfg.block_style == "parallel"
+        self.prepost = cfg.block_style == "prepost"
         self.layer_runs = cfg.layer_runs
-        if self.parallel:
+        if self.prepost:
+            if cfg.loop:
+                raise NotImplementedError("depth-averaged layers run once each")
+            W = cfg.hidden_size
+            self.pos = (nn.Parameter(torch.empty(cfg.max_position_embeddings, W, dtype=dtype, device=device))
+                        if cfg.pos_embed == "learned" else None)
+            self.layers = nn.ModuleList([PrePostBlock(cfg, spec, i + 2, dtype, device)
+                                         for i, spec in enumerate(cfg.layers)])
+            self.norm = nn.Parameter(torch.zeros(W, dtype=dtype, device=device))
+        elif self.parallel:
             blocks, seen_first = [], False
             for spec in cfg.layers:
                 v_mix = None
@@ -839,7 +1175,30 @@ class HybridDecoder(nn.Module):
         W = self.cfg.hidden_size
         for n, p in self.named_parameters():
             leaf = n.rsplit(".", 1)[-1]
-            if self.parallel:
+            if self.prepost:
+                if leaf == "dwa":  # mostly the layer's own result, a little of every earlier stream
+                    w = 0.3 * torch.rand(p.shape, generator=g) / p.shape[0]
+                    w[-1] = 1.0 - w[:-1].sum()
+                    p.data.copy_(w)
+                elif leaf == "sink":
+                    p.data.copy_(torch.randn(p.shape, generator=g))
+                elif leaf == "r1":
+                    p.data.copy_(0.2 + 0.6 * torch.rand(p.shape, generator=g))
+                elif leaf == "r2":
+                    p.data.copy_(0.1 + 0.9 * torch.rand(p.shape, generator=g))
+                elif leaf == "a2_bias":
+                    p.data.copy_(1.0 + torch.randn(p.shape, generator=g))
+                elif n.endswith("mix.norm") or leaf == "c_norm":  # plain weights
+                    p.data.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+                elif p.dim() == 1:  # norm weights stored around zero
+                    p.data.copy_(0.1 * torch.randn(p.shape, generator=g))
+                elif leaf == "pos":
+                    p.data.copy_(0.5 * torch.randn(p.shape, generator=g))
+                elif leaf == "embed":
+                    p.data.copy_(torch.randn(p.shape, generator=g))
+                else:
+                    p.data.copy_(torch.randn(p.shape, generator=g) / (p.shape[-1] ** 0.5))
+            elif self.parallel:
                 if leaf == "vmix":
                     p.data.copy_(0.2 + 0.6 * torch.rand(p.shape, generator=g))
                 elif leaf == "router_bias":
@@ -890,6 +1249,13 @@ class HybridDecoder(nn.Module):
     # ------------------------------------------------------------------------- checkpoint names
     def checkpoint_tensors(self) -> Dict[str, torch.Tensor]:
         """Checkpoint name -> the view of this model's parameters that holds it (fused projections are sliced)."""
+        if self.prepost:
+            out = {"embed": self.embed.data, "head": self.head.data, "final.norm": self.norm.data}
+            if self.pos is not None:
+                out["pos"] = self.pos.data
+            for i, blk in enumerate(self.layers):
+                out.update(blk.checkpoint_tensors(f"l{i}."))
+            return out
         if self.parallel:
             out = {"embed": self.embed.data, "final.norm": self.norm.data}
             for i, blk in enumerate(self.layers):

@@ -113,6 +113,34 @@ def moe_topk(logits: torch.Tensor, k: int, norm: bool, out_dtype=torch.float32):
     return topv, topi
 
 
+def moe_group_topk(logits: torch.Tensor, k: int, n_groups: int, keep: int):
+    """Sigmoid scores with group-limited choice, without autograd: logits fp32 [T, E]; the experts form `n_groups` equal
+    groups of neighbours, a group's score is the sum of its two largest sigmoid scores (of its only one for groups of
+    one), and the k largest scores among the members of the `keep` best groups are chosen. Returns (weights fp32 [T, k] =
+    the chosen scores as they are, expert ids int64 [T, k]), choices in descending order of score. One launch on the
+    GPU."""
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and E % n_groups == 0 and 1 <= keep <= n_groups and 1 <= k <= E
+    if L.use_hip(logits) and E <= 512 and k <= 64:
+        logits = logits.contiguous()
+        topi = torch.empty(T, k, dtype=torch.int64, device=logits.device)
+        topv = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        L.check(L.lib().areal_moe_group_topk(L.ptr(logits), L.c_int64(T), L.c_int(E), L.c_int(k), L.c_int(n_groups),
+                                             L.c_int(keep), L.ptr(topi), L.ptr(topv), L.stream_ptr()), "moe_group_topk")
+        return topv, topi
+    s = torch.sigmoid(logits)
+    masked = s
+    if n_groups > 1 and keep < n_groups:
+        gs = E // n_groups
+        grouped = s.view(T, n_groups, gs)
+        gscore = grouped.topk(min(2, gs), -1).values.sum(-1)
+        best = gscore.topk(keep, -1).indices
+        ok = torch.zeros(T, n_groups, dtype=torch.bool, device=s.device).scatter_(1, best, True)
+        masked = grouped.masked_fill(~ok.unsqueeze(-1), float("-inf")).view(T, E)
+    topv, topi = masked.topk(k, -1)
+    return torch.where(torch.isinf(topv), torch.zeros_like(topv), topv), topi
+
+
 def moe_sort(flat_e: torch.Tensor, n_experts: int, k: int):
     """Expert-sorted order of the (token, choice) pairs: flat_e int64 [T*k] with ids 0 .. n_experts (id n_experts =
     dropped pair, sorted last) -> (order [T*k], inv [T*k], src_row [T*k] = order // k, all int64; offsets int32

@@ -70,6 +70,35 @@ def qk_norm_cache_write(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_
     return q
 
 
+def qkv_vnorm_cache_write(proj: torch.Tensor, slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                          n_heads: int, eps: float, v_norm: bool = True) -> torch.Tensor:
+    """proj [T, >= (H + G) D + G Dv]: q heads | k heads | v heads (more columns may follow). Queries and keys stay as they
+    are; with `v_norm` every value head is divided by its root mean square over Dv (no weight) and is cached so. Writes
+    k and v of tokens with slot >= 0 into the paged caches and returns the queries [T, H, D] (contiguous)."""
+    T = proj.shape[0]
+    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[3]
+    H = n_heads
+    assert proj.stride(1) == 1 and proj.shape[1] >= (H + G) * D + G * V
+    q = torch.empty(T, H, D, dtype=proj.dtype, device=proj.device)
+    if L.use_hip(proj):
+        assert slots.dtype == torch.int64 and kcache.dtype == proj.dtype and vcache.dtype == proj.dtype
+        L.check(L.lib().areal_qkv_vnorm_cache_write(
+            L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(slots), L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.c_int(T),
+            L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_float(eps), L.c_int(int(v_norm)),
+            L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "qkv_vnorm_cache_write")
+        return q
+    q.copy_(proj[:, :H * D].reshape(T, H, D))
+    ok = slots >= 0
+    if ok.any():
+        pg, off = (slots[ok] // PAGE_SIZE).long(), (slots[ok] % PAGE_SIZE).long()
+        v = proj[ok, (H + G) * D:(H + G) * D + G * V].float().view(-1, G, V)
+        if v_norm:
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        kcache[pg, :, off, :] = proj[ok, H * D:(H + G) * D].view(-1, G, D)
+        vcache[pg, :, off, :] = v.to(vcache.dtype)
+    return q
+
+
 def rotation_table(base: float, dims: int, n_pos: int, device, scaling: Optional[dict] = None) -> torch.Tensor:
     """fp32 [n_pos, dims]: m cos(p f_i) for i < dims/2, then m sin(p f_i), with f_i = base^(-2i/dims).
 
@@ -210,10 +239,12 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                      cu_q: torch.Tensor, ctx_len: torch.Tensor, max_q: int, shape: ScoreShape,
                      mix: Optional[torch.Tensor] = None, nsplit: int = 1,
                      workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                     gate: Optional[torch.Tensor] = None, matrix_cores: bool = True) -> torch.Tensor:
+                     gate: Optional[torch.Tensor] = None, matrix_cores: bool = True,
+                     log_bias: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
     """q [T, H, D] (row b owns tokens cu_q[b]:cu_q[b+1], the LAST positions of its context of ctx_len[b] tokens,
     whose keys / values are in the cache already). mix [H, H] or None. gate [T, H] (a view with unit stride along
-    the heads) or None: head h of token t is multiplied by sigmoid(gate[t, h]). `matrix_cores`: bf16 rows of several
+    the heads) or None: head h of token t is multiplied by sigmoid(gate[t, h]); gate [T, H Dv]: one gate per value
+    channel. log_bias = (r1, r2), both [H]: r1_h ln(1 + r2_h (i - j)) is taken off the scaled score. `matrix_cores`: bf16 rows of several
     queries with head sizes 64 / 128, value sizes 32 / 64 / 128 and at most 16 heads (without `mix`: any number that
     splits into groups of whole key/value heads) run the MFMA kernel (False: always the plain one).
     Returns [T, H, Dv]."""
@@ -224,7 +255,13 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         assert q.is_contiguous() and kcache.dtype == q.dtype and block_tables.dtype == torch.int32
         assert cu_q.dtype == torch.int32 and ctx_len.dtype == torch.int32 and block_tables.is_contiguous()
         assert mix is None or (mix.dtype == q.dtype and mix.is_contiguous() and mix.shape == (H, H))
-        assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (T, H))
+        assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape in ((T, H), (T, H * V)))
+        gate_elem = gate is not None and gate.shape[1] == H * V and V > 1
+        r1 = r2 = None
+        if log_bias is not None:
+            r1, r2 = log_bias
+            assert r1.dtype == q.dtype and r2.dtype == q.dtype and r1.numel() == H and r2.numel() == H
+            assert r1.is_contiguous() and r2.is_contiguous()
         out = torch.empty(T, H, V, dtype=q.dtype, device=q.device)
         want = 1 if max_q == 1 else 16
         while want > 1 and want // 2 >= max_q:
@@ -242,7 +279,8 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
             assert pa.numel() >= T * nsplit * H * V and pm.numel() >= T * nsplit * H * 2
         L.check(L.lib().areal_window_attn(
             L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(cu_q),
-            L.ptr(ctx_len), L.ptr(mix), L.ptr(gate), L.c_int64(gate.stride(0) if gate is not None else 0), L.ptr(out),
+            L.ptr(ctx_len), L.ptr(mix), L.ptr(gate), L.c_int64(gate.stride(0) if gate is not None else 0),
+            L.c_int(int(gate_elem)), L.ptr(r1), L.ptr(r2), L.ptr(out),
             L.ptr(pa), L.ptr(pm), L.c_int(B), L.c_int(int(max_q)), L.c_int(T),
             L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_int(bq), L.c_float(shape.scale),
             L.c_float(shape.softcap), L.c_float(shape.slope_exp), L.c_int(int(shape.window)),
@@ -268,6 +306,9 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         i = torch.arange(ctx - n, ctx, device=q.device).view(n, 1)
         j = torch.arange(lo, ctx, device=q.device).view(1, -1)
         s = s - slopes.view(H, 1, 1) * (i - j).float()
+        if log_bias is not None:
+            s = s - log_bias[0].float().view(H, 1, 1) * torch.log1p(log_bias[1].float().view(H, 1, 1)
+                                                                      * (i - j).clamp(min=0).float())
         if mix is not None:
             s = torch.einsum("hg,gij->hij", mix.float(), s)
         ok = (i - j >= 0) & (((i - j < shape.window) | (j < shape.keep_first)) if shape.window > 0 else True)
@@ -279,5 +320,6 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         den = e.sum(-1, keepdim=True) + (torch.exp(-m) if shape.sink else 0.0)
         out[cq[b]:cq[b + 1]] = torch.einsum("hij,hjv->ihv", e / den, vv)
     if gate is not None:
-        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
+        g = torch.sigmoid(gate.float())
+        out = out * (g.view(T, H, V) if gate.shape[1] == H * V and V > 1 else g.unsqueeze(-1))
     return out.to(q.dtype)

@@ -15,7 +15,10 @@
 // The same kernel serves prompt portions (grid x = query tiles x head groups, y = rows of the batch) and decoding
 // (BQ = 1, grid z = splits of the visible key range whose partial results `latent_attn_combine` merges).
 // Queries of row b are the LAST cu_q[b+1] - cu_q[b] positions of its context of ctx_len[b] tokens.
-// Rotation: pairs (i, i + P/2); table [n_pos][P] = cos | sin of position * frequency.
+// Rotation: pairs (i, i + P/2), or (`neighbours`) pairs (2i, 2i + 1) of the projection's columns; table [n_pos][P] =
+// cos | sin of position * frequency. Rotated neighbour pairs are stored (cache) and scored (query) in the order
+// first members | second members: a dot product does not see a permutation applied to both of its sides.
+// `sink` (one logit per head, or null): a key without a value whose exp(sink_h) counts once in the denominator.
 #include "common.hpp"
 
 namespace {
@@ -34,12 +37,13 @@ template <typename T>
 __global__ void __launch_bounds__(256) latent_prep_kernel(
     const T* __restrict__ proj, int64_t row_stride, const T* __restrict__ qw, const T* __restrict__ cw,
     const int* __restrict__ positions, const int64_t* __restrict__ slots, const float* __restrict__ table, int n_pos,
-    T* __restrict__ cq, T* __restrict__ cache, int Q, int R, int P, float eps) {
+    T* __restrict__ cq, T* __restrict__ cache, int Q, int R, int P, float eps, int neighbours) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = proj + (size_t)t * row_stride;
   const int64_t slot = slots[t];
   T* dst = slot >= 0 ? cache + (size_t)slot * (R + P) : nullptr;  // slot = page * 32 + offset
   if (wave == 0) {
+    if (Q <= 0) return;
     float ss = 0.f;
     for (int i = lane; i < Q; i += 64) {
       const float x = ldf<T>(row, i);
@@ -62,7 +66,8 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(
     const float* cs = table + (size_t)pos * P;
     const int half = P / 2;
     for (int i = lane; i < half; i += 64) {
-      const float u = ldf<T>(row, Q + R + i), v = ldf<T>(row, Q + R + half + i);
+      const float u = ldf<T>(row, Q + R + (neighbours ? 2 * i : i));
+      const float v = ldf<T>(row, Q + R + (neighbours ? 2 * i + 1 : half + i));
       const float c = cs[i], s = cs[half + i];
       stf<T>(dst, R + i, u * c - v * s);
       stf<T>(dst, R + half + i, v * c + u * s);
@@ -81,9 +86,10 @@ struct LatentShape {
 
 template <typename T>
 __global__ void __launch_bounds__(256) latent_attn_kernel(
-    const T* __restrict__ q, const T* __restrict__ q_lat, const T* __restrict__ cache,
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ q_lat, const T* __restrict__ cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const T* __restrict__ gate,
+    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, int neighbours,
+    const T* __restrict__ sink, const T* __restrict__ gate,
     int64_t gate_stride, T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     LatentShape sh, float scale, int window, int nsplit) {
   extern __shared__ float lds[];
@@ -118,9 +124,10 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
         v = ldf<T>(q_lat, (tok * H + h0 + hh) * R + d);
       } else {
         const int e = d - R, pi = e < half ? e : e - half;
-        const T* qr = q + (tok * H + h0 + hh) * (D + P) + D;
+        const T* qr = q + tok * q_stride + (size_t)(h0 + hh) * (D + P) + D;
         const float* cs = table + (size_t)min(max(pos0 + qi, 0), n_pos - 1) * P;
-        const float u = ldf<T>(qr, pi), w = ldf<T>(qr, half + pi), c = cs[pi], s = cs[half + pi];
+        const float u = ldf<T>(qr, neighbours ? 2 * pi : pi), w = ldf<T>(qr, neighbours ? 2 * pi + 1 : half + pi);
+        const float c = cs[pi], s = cs[half + pi];
         v = e < half ? u * c - w * s : w * c + u * s;
       }
     }
@@ -128,8 +135,10 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
   }
   for (int i = tid; i < NR * R; i += 256) acc[i] = 0.f;
   for (int i = tid; i < NR; i += 256) {
-    mrow[i] = -1e30f;
-    lrow[i] = 0.f;
+    const int hh = i / BQ;
+    const bool with_sink = sink && split == 0 && hh < nh;
+    mrow[i] = with_sink ? ldf<T>(sink, h0 + hh) : -1e30f;
+    lrow[i] = with_sink ? 1.f : 0.f;
   }
 
   // visible keys of the tile: [j_lo, j_hi); pages [p_lo, p_hi), this split's share of them
@@ -236,9 +245,10 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
 // KW32 = (R + P) / 32 k-steps of the scores, R16 = R / 16 output tiles.
 template <int KW32, int R16, int RS, bool DEC>
 __global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ cache,
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const bf16_t* __restrict__ gate,
+    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, int neighbours,
+    const bf16_t* __restrict__ sink, const bf16_t* __restrict__ gate,
     int64_t gate_stride, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
     int HG, int D, float scale, int window, int nsplit) {
   constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 4, SS = PAGE + 4, NT = R16 / RS;
@@ -280,8 +290,10 @@ __global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
   float mrow[4], lrow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    mrow[i] = -1e30f;
-    lrow[i] = 0.f;
+    const int r = 4 * quad + i;
+    const bool with_sink = sink && split == 0 && r < nrows;
+    mrow[i] = with_sink ? bf2f(sink[row_head(r)]) : -1e30f;
+    lrow[i] = with_sink ? 1.f : 0.f;
   }
 #pragma unroll
   for (int vt = 0; vt < NT; ++vt) acc[vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -296,8 +308,16 @@ __global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
       } else {  // rotary part: entry e pairs with e +- P/2
         constexpr int half = P / 2;
         const int e = d - R, pi = e < half ? e : e - half;
-        const bf16_t* qr = q + (tok * H + h) * (size_t)(D + P) + D;
-        const bf16x8 u = ld8(qr + pi), w = ld8(qr + half + pi);
+        const bf16_t* qr = q + tok * q_stride + (size_t)h * (D + P) + D;
+        bf16x8 u, w;
+        if (neighbours) {  // 16 consecutive columns hold the 8 pairs
+          const bf16x8 x0 = ld8(qr + 2 * pi), x1 = ld8(qr + 2 * pi + 8);
+          u = (bf16x8){x0[0], x0[2], x0[4], x0[6], x1[0], x1[2], x1[4], x1[6]};
+          w = (bf16x8){x0[1], x0[3], x0[5], x0[7], x1[1], x1[3], x1[5], x1[7]};
+        } else {
+          u = ld8(qr + pi);
+          w = ld8(qr + half + pi);
+        }
         const float* cs = table + (size_t)min(max(row_pos(r16), 0), n_pos - 1) * P;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
@@ -463,14 +483,17 @@ size_t mfma_lds_bytes(int R, int P, int waves) {
 }
 
 // Shapes the matrix-core kernel is instantiated for: (latent size, rotary size), unrotated key size D.
-bool mfma_usable(int R, int P, int D) {
-  if (D % 8 != 0) return false;  // 16-byte loads of the rotary query part
+bool mfma_usable(int R, int P, int D, int64_t q_stride) {
+  if (D % 8 != 0 || q_stride % 8 != 0) return false;  // 16-byte loads of the rotary query part
   return (R == 512 && P == 64) || (R == 256 && (P == 64 || P == 32)) || (R == 128 && (P == 64 || P == 32)) ||
          (R == 64 && (P == 64 || P == 32));
 }
 
 struct MfmaArgs {
   const bf16_t *q, *q_lat, *cache;
+  int64_t q_stride;
+  int neighbours;
+  const bf16_t* sink;
   const int* bt;
   int max_pages;
   const int *cu_q, *ctx_len;
@@ -494,8 +517,9 @@ int launch_mfma(dim3 grid, int nthr, int hg, hipStream_t st, const MfmaArgs& a) 
     raised = true;
   }
   const size_t lds = mfma_lds_bytes(R16 * 16, KW32 * 32 - R16 * 16, DEC ? 1 : nthr / 64);
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16, RS, DEC>), grid, dim3(nthr), lds, st, a.q, a.q_lat, a.cache,
-                     a.bt, a.max_pages, a.cu_q, a.ctx_len, a.table, a.n_pos, a.gate, a.gate_stride, a.out, a.part_acc,
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16, RS, DEC>), grid, dim3(nthr), lds, st, a.q, a.q_stride, a.q_lat,
+                     a.cache, a.bt, a.max_pages, a.cu_q, a.ctx_len, a.table, a.n_pos, a.neighbours, a.sink, a.gate,
+                     a.gate_stride, a.out, a.part_acc,
                      a.part_ml, a.H, hg, a.D, a.scale, a.window, a.nsplit);
   return (int)hipGetLastError();
 }
@@ -576,32 +600,35 @@ bool pick_shape(int H, int D, int P, int R, int want, LatentShape* out) {
 
 extern "C" int areal_latent_prep(const void* proj, int64_t row_stride, const void* qw, const void* cw,
                                  const int* positions, const int64_t* slots, const float* table, int n_pos, void* cq,
-                                 void* cache, int T, int Q, int R, int P, float eps, int dt, hipStream_t st) {
+                                 void* cache, int T, int Q, int R, int P, float eps, int neighbours, int dt,
+                                 hipStream_t st) {
   if (T == 0) return 0;
   if (P % 2 || n_pos < 1) return -1;
   if (dt == 0)
     hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
                        (const bf16_t*)qw, (const bf16_t*)cw, positions, slots, table, n_pos, (bf16_t*)cq,
-                       (bf16_t*)cache, Q, R, P, eps);
+                       (bf16_t*)cache, Q, R, P, eps, neighbours);
   else
     hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
                        (const float*)qw, (const float*)cw, positions, slots, table, n_pos, (float*)cq, (float*)cache,
-                       Q, R, P, eps);
+                       Q, R, P, eps, neighbours);
   return (int)hipGetLastError();
 }
 
 // B rows; row b's queries are tokens cu_q[b] .. cu_q[b+1]; max_q = longest row. nsplit > 1 needs part_acc
 // [T, nsplit, H, R] and part_ml [T, nsplit, H, 2] (fp32) and is meant for single-query rows.
-extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* cache, const int* block_tables,
-                                 int max_pages, const int* cu_q, const int* ctx_len, const float* table, int n_pos,
-                                 const void* gate, int64_t gate_stride, void* out, float* part_acc, float* part_ml,
+extern "C" int areal_latent_attn(const void* q, int64_t q_stride, const void* q_lat, const void* cache,
+                                 const int* block_tables, int max_pages, const int* cu_q, const int* ctx_len,
+                                 const float* table, int n_pos, int neighbours, const void* sink, const void* gate, int64_t gate_stride, void* out, float* part_acc, float* part_ml,
                                  int B, int max_q, int T, int H, int D, int P, int R, float scale, int window,
                                  int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (H < 1 || R < 1 || P % 2 || nsplit < 1 || nsplit > 64 || n_pos < 1) return -1;
   if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
-  if (matrix_cores && dt == 0 && mfma_usable(R, P, D) && (max_q > 1 ? nsplit == 1 : true)) {
-    const MfmaArgs a{(const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, block_tables, max_pages, cu_q,
+  if (matrix_cores && dt == 0 && mfma_usable(R, P, D, q_stride) && ((uintptr_t)q % 16) == 0 &&
+      (max_q > 1 ? nsplit == 1 : true)) {
+    const MfmaArgs a{(const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, q_stride, neighbours,
+                     (const bf16_t*)sink, block_tables, max_pages, cu_q,
                      ctx_len, table, n_pos, (const bf16_t*)gate, gate_stride, (bf16_t*)out, part_acc, part_ml, H, D,
                      scale, window, nsplit};
     if (max_q > 1) return dispatch_mfma<false>(R, P, B, max_q, st, a);
@@ -626,9 +653,9 @@ extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* c
                                   160 * 1024));                                                                     \
       allowed = 160 * 1024;                                                                                         \
     }                                                                                                               \
-    hipLaunchKernelGGL(latent_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)q_lat,            \
-                       (const TT*)cache, block_tables, max_pages, cu_q, ctx_len, table, n_pos, (const TT*)gate,     \
-                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, window, nsplit);                        \
+    hipLaunchKernelGGL(latent_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, q_stride, (const TT*)q_lat,  \
+                       (const TT*)cache, block_tables, max_pages, cu_q, ctx_len, table, n_pos, neighbours,          \
+                       (const TT*)sink, (const TT*)gate, gate_stride, (TT*)out, part_acc, part_ml, sh, scale, window, nsplit);                        \
     if (nsplit > 1)                                                                                                 \
       hipLaunchKernelGGL(latent_attn_combine_kernel<TT>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,           \
                          (const TT*)gate, gate_stride, (TT*)out, H, R, nsplit);                                     \

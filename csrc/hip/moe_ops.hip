@@ -387,6 +387,141 @@ extern "C" int areal_moe_topk(const void* logits, int dtype, int64_t T, int E, i
   return topk_launch((const float*)logits, T, E, k, norm, topi, topv, (bf16_t*)topv_bf, st);
 }
 
+// Sigmoid scores with group-limited choice: the E experts form `n_groups` equal groups of neighbours, a group's score is
+// the sum of its two largest sigmoid scores (of its only one, for groups of one), and the k experts with the largest
+// scores are taken among the members of the `keep` best groups (value descending, index ascending on ties). The
+// weights are the chosen scores themselves. One wave (= one workgroup) per token.
+template <int PER_LANE>
+__global__ __launch_bounds__(64) void moe_group_topk_kernel(const float* __restrict__ logits, int E, int k,
+                                                            int n_groups, int keep, int64_t* __restrict__ topi,
+                                                            float* __restrict__ topv) {
+  __shared__ float sc[64 * PER_LANE];
+  __shared__ float gsc[64 * PER_LANE];
+  __shared__ int okf[64 * PER_LANE];
+  const int lane = threadIdx.x;
+  const int64_t t = blockIdx.x;
+  const float* row = logits + t * (int64_t)E;
+  float v[PER_LANE];
+#pragma unroll
+  for (int i = 0; i < PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < E ? 1.f / (1.f + expf(-row[e])) : -INFINITY;
+    sc[e] = v[i];
+    okf[e] = 0;
+  }
+  if (n_groups > 1 && keep < n_groups) {
+    const int gs = E / n_groups;
+    __syncthreads();
+    for (int g = lane; g < n_groups; g += 64) {
+      float m1 = -INFINITY, m2 = -INFINITY;
+      for (int j = 0; j < gs; ++j) {
+        const float x = sc[g * gs + j];
+        if (x > m1) {
+          m2 = m1;
+          m1 = x;
+        } else if (x > m2) {
+          m2 = x;
+        }
+      }
+      gsc[g] = gs > 1 ? m1 + m2 : m1;
+    }
+    __syncthreads();
+    float gv[PER_LANE];
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) gv[i] = lane + 64 * i < n_groups ? gsc[lane + 64 * i] : -INFINITY;
+    for (int j = 0; j < keep; ++j) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+#pragma unroll
+      for (int i = 0; i < PER_LANE; ++i) {
+        if (gv[i] > bv) {
+          bv = gv[i];
+          bi = lane + 64 * i;
+        }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (bi >= n_groups) break;
+      if ((bi & 63) == lane) {
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i)
+          if (i == (bi >> 6)) gv[i] = -INFINITY;
+        okf[bi] = 1;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && !okf[e / gs]) v[i] = -INFINITY;
+    }
+  }
+  float mine_v = 0.f;  // lane j keeps choice j
+  int mine_i = 0;
+  for (int j = 0; j < k; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+      if (v[i] > bv) {
+        bv = v[i];
+        bi = lane + 64 * i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi >= E) {  // fewer eligible experts than k: the remaining choices carry no weight
+      bi = 0;
+      bv = 0.f;
+    }
+    if (lane == j) {
+      mine_v = bv;
+      mine_i = bi;
+    }
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < PER_LANE; ++i)
+        if (i == (bi >> 6)) v[i] = -INFINITY;
+    }
+  }
+  if (lane < k) {
+    topi[t * k + lane] = mine_i;
+    topv[t * k + lane] = mine_v;
+  }
+}
+
+// logits fp32 [T, E]; n_groups divides E; 1 <= keep <= n_groups. topi int64 [T, k], topv fp32 [T, k].
+extern "C" int areal_moe_group_topk(const float* logits, int64_t T, int E, int k, int n_groups, int keep, int64_t* topi,
+                                    float* topv, hipStream_t st) {
+  if (T == 0) return 0;
+  if (E < 1 || E > 64 * RT_MAX_PER_LANE || k < 1 || k > 64 || k > E || n_groups < 1 || E % n_groups != 0 || keep < 1 ||
+      keep > n_groups)
+    return -1;
+  const dim3 grid((unsigned)T), block(64);
+#define GT_CASE(P)                                                                                                 \
+  if (E <= 64 * P) {                                                                                               \
+    hipLaunchKernelGGL((moe_group_topk_kernel<P>), grid, block, 0, st, logits, E, k, n_groups, keep, topi, topv);  \
+    return (int)hipGetLastError();                                                                                 \
+  }
+  GT_CASE(1) GT_CASE(2) GT_CASE(4) GT_CASE(8)
+#undef GT_CASE
+  return -1;
+}
+
 // Largest list the one-workgroup sort takes (its slice x bin table has to fit 64 KiB of LDS for every bin count up
 // to the maximum); chunks of the three-launch form hold `items` tiles of 256 pairs.
 static bool sort_single_fits(int64_t n, int bins) {

@@ -3,11 +3,13 @@
 //   s_g(i, j)  = (q_g(i) . k_c(g)(j)) * scale                      c(g) = g / (H / G): grouped key/value heads
 //   s_g       <- cap * tanh(s_g / cap)                             (cap > 0; otherwise left as it is)
 //   s_g       <- s_g - slope_g * (i - j),  slope_g = 2^(-slope_exp * (g + 1) / H)     (slope_exp = 0: no bias)
+//   s_g       <- s_g - r1_g * ln(1 + r2_g * (i - j))              (r1 / r2 given: a learned logarithmic distance penalty)
 //   t_h        = sum_g M[h, g] s_g                                 head mixing (M = null: t_h = s_h)
 //   visible:     0 <= i - j < window, or j <= i and j < keep_first    (window <= 0: every earlier key; the first
 //                keep_first tokens of a sequence stay visible to every later query, at their true positions)
 //   p_h(j)     = exp(t_h(j)) / (sink + sum_j' exp(t_h(j')))        sink = 1: a key of score 0 that has no value
-//   o_h(i)     = sum_j p_h(j) v_c(h)(j)  [* sigmoid(gate_h(i)) when a gate is given: one number per head and token]
+//   o_h(i)     = sum_j p_h(j) v_c(h)(j)  [* sigmoid(gate_h(i)) when a gate is given: one number per head and token, or
+//                one per head, token and value channel (`gate_elem`)]
 //
 // Scores, weights and the accumulation run in fp32 whatever the storage type T (bf16 / fp32) of q, the caches
 // and the output. Because the heads are mixed before the softmax, one workgroup owns ALL heads of a tile of BQ
@@ -216,6 +218,45 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_vec_kernel(
   }
 }
 
+// Per token: queries and keys as they are (queries -> q_out, keys -> K cache); every value head divided by its root
+// mean square over its V elements (no weight; `v_norm` = 0: copied) -> V cache. One head a wave, a token's heads
+// spread over grid y.
+template <typename T>
+__global__ void __launch_bounds__(256) qkv_vnorm_cache_write_kernel(
+    const T* __restrict__ proj, int64_t row_stride, const int64_t* __restrict__ slots, T* __restrict__ q_out,
+    T* __restrict__ kcache, T* __restrict__ vcache, int H, int G, int D, int V, float eps, int v_norm) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * row_stride;
+  const int64_t slot = slots[t];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t page = slot >= 0 ? (size_t)(slot / PAGE) : 0;
+  const int off = slot >= 0 ? (int)(slot % PAGE) : 0;
+  for (int u = blockIdx.y * 4 + wave; u < H + 2 * G; u += 4 * gridDim.y) {
+    if (u < H) {
+      for (int d = lane; d < D; d += 64) q_out[((size_t)t * H + u) * D + d] = row[(size_t)u * D + d];
+    } else if (slot < 0) {
+      continue;
+    } else if (u < H + G) {
+      T* dst = kcache + ((page * G + (u - H)) * PAGE + off) * D;
+      for (int d = lane; d < D; d += 64) dst[d] = row[(size_t)u * D + d];
+    } else {
+      const int c = u - H - G;
+      const T* src = row + (size_t)(H + G) * D + (size_t)c * V;
+      T* dst = vcache + ((page * G + c) * PAGE + off) * V;
+      float r = 1.f;
+      if (v_norm) {
+        float ss = 0.f;
+        for (int d = lane; d < V; d += 64) {
+          const float x = ldf<T>(src, d);
+          ss += x * x;
+        }
+        r = 1.f / sqrtf(wave_sum(ss) / (float)V + eps);
+      }
+      for (int d = lane; d < V; d += 64) stf<T>(dst, d, v_norm ? ldf<T>(src, d) * r : ldf<T>(src, d));
+    }
+  }
+}
+
 struct AttnShape {
   int H, G, D, V, BQ;
   // LDS layout in floats
@@ -231,6 +272,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     const T* __restrict__ q, const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const T* __restrict__ mix, const T* __restrict__ gate, int64_t gate_stride,
+    int gate_elem, const T* __restrict__ r1, const T* __restrict__ r2,
     T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int keep, int sink,
     int nsplit) {
   extern __shared__ float lds[];
@@ -305,6 +347,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
         s *= scale;
         if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         if (slope_exp != 0.f) s -= exp2f(-slope_exp * (float)(g + 1) / (float)H) * (float)(pos0 + qi - (jb + kj));
+        if (r1) s -= ldf<T>(r1, g) * log1pf(ldf<T>(r2, g) * (float)max(pos0 + qi - (jb + kj), 0));
         S1[((size_t)g * BQ + qi) * PAGE + kj] = s;
       }
     }
@@ -377,7 +420,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     if (nsplit == 1) {
       const float l = lrow[r];
       float val = l > 0.f ? acc[o] / l : 0.f;
-      if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+      if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + (gate_elem ? h * V + v : h)));
       stf<T>(out, (tok * H + h) * V + v, val);
     } else {
       part_acc[((tok * nsplit + split) * H + h) * V + v] = acc[o];
@@ -405,7 +448,8 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const bf16_t* __restrict__ mix, const bf16_t* __restrict__ gate,
-    int64_t gate_stride, bf16_t* __restrict__ out, int Hall, int Gall, int H, float scale, float softcap,
+    int64_t gate_stride, int gate_elem, const bf16_t* __restrict__ r1, const bf16_t* __restrict__ r2,
+    bf16_t* __restrict__ out, int Hall, int Gall, int H, float scale, float softcap,
     float slope_exp, int window, int keep, int sink) {
   constexpr int D = DK * 32, V = VT_ * 16, KS = D + 8, VS = PAGE + 8, SS = PAGE + 4;
   // this workgroup's heads: hbase .. hbase + H - 1 of Hall (several groups only without head mixing), and their G
@@ -437,11 +481,13 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
   }
   bf16x8 qf[HPW][DK];
   f32x4 acc[HPW][VT_];
-  float slope[HPW];
+  float slope[HPW], lr1[HPW], lr2[HPW];
 #pragma unroll
   for (int hh = 0; hh < HPW; ++hh) {
     const int h = wave * HPW + hh;
     slope[hh] = slope_exp != 0.f ? exp2f(-slope_exp * (float)(hbase + h + 1) / (float)Hall) : 0.f;
+    lr1[hh] = r1 ? bf2f(r1[hbase + h]) : 0.f;
+    lr2[hh] = r1 ? bf2f(r2[hbase + h]) : 0.f;
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks) {
       if (r16 < nq) qf[hh][ks] = ld8(q + ((size_t)(q0 + t0 + r16) * Hall + hbase + h) * D + 32 * ks + 8 * quad);
@@ -496,6 +542,7 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
             sc = softcap * ((e - 1.f) / (e + 1.f));
           }
           sc -= slope[hh] * (float)(pos0 + qi - (jb + 16 * half + r16));
+          if (r1) sc -= lr1[hh] * __logf(1.f + lr2[hh] * (float)max(pos0 + qi - (jb + 16 * half + r16), 0));
           SM[((size_t)h * 16 + qi) * SS + 16 * half + r16] = __float_as_uint(sc);
         }
       }
@@ -577,9 +624,13 @@ __global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
       const size_t tok = (size_t)(q0 + t0 + qi);
       const float l = lS[h * 16 + qi];
       float f = l > 0.f ? 1.f / l : 0.f;
-      if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + hbase + h]));
+      if (gate && !gate_elem) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + hbase + h]));
 #pragma unroll
-      for (int vt = 0; vt < VT_; ++vt) out[(tok * Hall + hbase + h) * V + 16 * vt + r16] = f2bf(acc[hh][vt][i] * f);
+      for (int vt = 0; vt < VT_; ++vt) {
+        float val = acc[hh][vt][i] * f;
+        if (gate && gate_elem) val /= 1.f + expf(-bf2f(gate[tok * gate_stride + (size_t)(hbase + h) * V + 16 * vt + r16]));
+        out[(tok * Hall + hbase + h) * V + 16 * vt + r16] = f2bf(val);
+      }
     }
   }
 }
@@ -608,8 +659,9 @@ bool mfma_usable(int H, int G, int D, int V, bool mixed) {
 template <int HPW, int MAXT>
 int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* kc, const bf16_t* vc,
                 const int* bt, int max_pages, const int* cu_q, const int* ctx_len, const bf16_t* mix,
-                const bf16_t* gate, int64_t gate_stride, bf16_t* out, int Hall, int Gall, int H, int D, int V,
-                float scale, float softcap, float slope_exp, int window, int keep, int sink) {
+                const bf16_t* gate, int64_t gate_stride, int gate_elem, const bf16_t* r1, const bf16_t* r2, bf16_t* out,
+                int Hall, int Gall, int H, int D, int V, float scale, float softcap, float slope_exp, int window,
+                int keep, int sink) {
 #define MFMA_CASE(DKV, VTV)                                                                                        \
   do {                                                                                                             \
     static bool raised = false; /* once per kernel: no attribute call inside a stream capture later */            \
@@ -619,8 +671,8 @@ int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q
       raised = true;                                                                                               \
     }                                                                                                              \
     hipLaunchKernelGGL((window_attn_mfma_kernel<HPW, DKV, VTV, MAXT>), grid, dim3(nthr), lds, st, q, kc, vc, bt,   \
-                       max_pages, cu_q, ctx_len, mix, gate, gate_stride, out, Hall, Gall, H, scale, softcap,       \
-                       slope_exp, window, keep, sink);                                                             \
+                       max_pages, cu_q, ctx_len, mix, gate, gate_stride, gate_elem, r1, r2, out, Hall, Gall, H,    \
+                       scale, softcap, slope_exp, window, keep, sink);                                             \
   } while (0)
   if (D == 64 && V == 32) MFMA_CASE(2, 2);
   else if (D == 64 && V == 64) MFMA_CASE(2, 4);
@@ -637,7 +689,8 @@ template <typename T>
 __global__ void __launch_bounds__(128) window_attn_combine_kernel(const float* __restrict__ part_acc,
                                                                    const float* __restrict__ part_ml,
                                                                    const T* __restrict__ gate, int64_t gate_stride,
-                                                                   T* __restrict__ out, int H, int V, int nsplit) {
+                                                                   int gate_elem, T* __restrict__ out, int H, int V,
+                                                                   int nsplit) {
   const size_t tok = blockIdx.x;
   const int h = blockIdx.y;
   float M = -1e30f;
@@ -646,12 +699,14 @@ __global__ void __launch_bounds__(128) window_attn_combine_kernel(const float* _
   for (int s = 0; s < nsplit; ++s)
     den += expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M) * part_ml[((tok * nsplit + s) * H + h) * 2 + 1];
   float f = den > 0.f ? 1.f / den : 0.f;
-  if (gate) f /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+  if (gate && !gate_elem) f /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
   for (int v = threadIdx.x; v < V; v += 128) {
     float num = 0.f;
     for (int s = 0; s < nsplit; ++s)
       num += expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M) * part_acc[((tok * nsplit + s) * H + h) * V + v];
-    stf<T>(out, (tok * H + h) * V + v, num * f);
+    num *= f;
+    if (gate && gate_elem) num /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + (size_t)h * V + v));
+    stf<T>(out, (tok * H + h) * V + v, num);
   }
 }
 
@@ -705,6 +760,21 @@ extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, 
   return (int)hipGetLastError();
 }
 
+// proj rows: q heads | k heads | v heads from the pointer on; nothing is rotated or normed but (v_norm) the values
+extern "C" int areal_qkv_vnorm_cache_write(const void* proj, int64_t row_stride, const int64_t* slots, void* q_out,
+                                           void* kcache, void* vcache, int T, int H, int G, int D, int V, float eps,
+                                           int v_norm, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  const dim3 grid(T, (H + 2 * G + 3) / 4);
+  if (dt == 0)
+    hipLaunchKernelGGL(qkv_vnorm_cache_write_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)proj, row_stride,
+                       slots, (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_norm);
+  else
+    hipLaunchKernelGGL(qkv_vnorm_cache_write_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, row_stride,
+                       slots, (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps, v_norm);
+  return (int)hipGetLastError();
+}
+
 // Largest query tile (16, 8, 4, 2, 1) whose LDS footprint fits the workgroup limit; 0 if even one query does not.
 extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
   for (int bq = want; bq >= 1; bq >>= 1) {
@@ -718,11 +788,12 @@ extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
 // part_acc [T, nsplit, H, V] and part_ml [T, nsplit, H, 2] (fp32) and is meant for single-query rows.
 extern "C" int areal_window_attn(const void* q, const void* kcache, const void* vcache, const int* block_tables,
                                  int max_pages, const int* cu_q, const int* ctx_len, const void* mix, const void* gate,
-                                 int64_t gate_stride, void* out, float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
+                                 int64_t gate_stride, int gate_elem, const void* r1, const void* r2, void* out,
+                                 float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
                                  int bq, float scale, float softcap, float slope_exp, int window, int keep, int sink,
                                  int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
-  if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1) return -1;
+  if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1 || (r1 == nullptr) != (r2 == nullptr)) return -1;
   if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(H, G, D, V, mix != nullptr)) {
     const int hb = mfma_head_group(H, G, mix != nullptr);
     const int hpw = mfma_heads_per_wave(hb), nthr = 64 * (hb / hpw);
@@ -730,8 +801,8 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
     const size_t mlds = mfma_lds_bytes(hb / (H / G), D, V);
 #define MFMA_ARGS                                                                                                  \
   mgrid, nthr, mlds, st, (const bf16_t*)q, (const bf16_t*)kcache, (const bf16_t*)vcache, block_tables, max_pages,   \
-      cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, G, hb, D, V, scale,      \
-      softcap, slope_exp, window, keep, sink
+      cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, gate_elem, (const bf16_t*)r1,            \
+      (const bf16_t*)r2, (bf16_t*)out, H, G, hb, D, V, scale, softcap, slope_exp, window, keep, sink
     if (hpw == 4) return launch_mfma<4, 256>(MFMA_ARGS);
     if (hpw == 2) return launch_mfma<2, 512>(MFMA_ARGS);
     return launch_mfma<1, 512>(MFMA_ARGS);
@@ -752,11 +823,11 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
     }                                                                                                                \
     hipLaunchKernelGGL(window_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)kcache,            \
                        (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (const TT*)gate,   \
-                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, softcap, slope_exp, window, keep, sink,   \
-                       nsplit);                                                                                     \
+                       gate_stride, gate_elem, (const TT*)r1, (const TT*)r2, (TT*)out, part_acc, part_ml, sh, scale, \
+                       softcap, slope_exp, window, keep, sink, nsplit);                                             \
     if (nsplit > 1)                                                                                                  \
       hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,           \
-                         (const TT*)gate, gate_stride, (TT*)out, H, V, nsplit);                                      \
+                         (const TT*)gate, gate_stride, gate_elem, (TT*)out, H, V, nsplit);                          \
   } while (0)
   if (dt == 0) LAUNCH(bf16_t);
   else LAUNCH(float);
