@@ -167,3 +167,13 @@ def forward(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], tokens: List[int]):
         x = sum(w[p + "dwa"][j] * stack[j] for j in range(i + 2))
         after.append(x)
     return norm_centered(x, w["final.norm"], eps) @ w["head"].T, torch.stack(after)
+
+
+def greedy(cfg: Dict[str, Any], w: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
+    """Greedy continuation, recomputing the whole sequence for every new token."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        logits, _ = forward(cfg, w, toks)
+        out.append(int(torch.argmax(logits[-1])))
+        toks.append(out[-1])
+    return out
