@@ -696,7 +696,7 @@ def test_random_shapes_orders_and_schedules(device, dtype, seed):
                 layers.append(gla(rng.choice([1, 2, 3]), rng.choice([8, 24, 64, 128]), rng.choice([8, 40, 64, 72]),
                                   rng.choice([1.0, 4.0, 16.0]), rng.choice([1, 4, 16]), mlp))
         cfg = config(layers, width=width, vocab=vocab, eps=rng.choice([1e-5, 1e-6]), mult=rng.choice([0.2, 1.0]))
-        reqs = {f"q{i}": tokens_of(rng.choice([1, 2, 17, 97, 150]), vocab, 100 * case + i)
+        reqs = {f"q{i}": tokens_of(rng.choice([1, 2, 17, 97, 150]), vocab, 7 + 100 * case + i)
                 for i in range(rng.randint(1, 3))}
         at, steps = {r: 0 for r in reqs}, []
         while any(at[r] < len(t) for r, t in reqs.items()):
