@@ -13,6 +13,10 @@ per token, its experts as wide as the parameter budget allows.
 The Pobelorn design (parallel blocks; window attention on rotated unit-norm queries and keys that keeps the first
 tokens, every third layer lightning attention; routed + shared gated experts, the first layer a squared-ReLU MLP) is
 compared with the same kind of twin.
+
+The Zusotar design (sublayers between two RMS norms, a learned average over depth; window attention with a logarithmic
+distance penalty, latent attention with a sink and gated linear attention in turn; group-routed + shared gated
+experts, the first layer a gated MLP) is compared with the same kind of twin.
 """
 import json
 import sys
@@ -40,6 +44,14 @@ POBELORN_SIZES = {
     "w1024": (1024, 4, 8, 2, 128, 64, 512, 4, 16, 2, 512, 512),
     "w2048": (2048, 4, 16, 4, 128, 64, 1024, 4, 32, 4, 768, 768),
     "w4096": (4096, 2, 32, 8, 128, 64, 1024, 4, 64, 4, 1024, 1024),
+}
+# Zusotar: width, layers, heads, kv heads, head size of the window attention (keys, values), window, latent attention's
+# unrotated / rotary / value size per head and latent size, gla heads / key size / value size / decay rank, experts,
+# experts per token, groups, groups kept, expert width, shared expert width
+ZUSOTAR_SIZES = {
+    "w1024": (1024, 4, 8, 2, 128, 512, 64, 32, 64, 256, 4, 128, 256, 16, 16, 2, 4, 2, 512, 512),
+    "w2048": (2048, 4, 16, 4, 128, 1024, 128, 64, 128, 512, 8, 128, 256, 16, 32, 4, 4, 2, 768, 768),
+    "w4096": (4096, 3, 32, 8, 128, 1024, 128, 64, 128, 512, 16, 128, 256, 32, 64, 4, 8, 4, 1024, 1024),
 }
 VOCAB = 32768
 
@@ -86,6 +98,26 @@ def pobelorn_dict(width, layers, heads, kv, dim, rot, window, keep, experts, top
                                          "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}})
     return {"architecture": "Pobelorn", "embedding": {"scale": float(width) ** 0.5}, "layers": ls, "norm": {"eps": 1e-6},
             "vocab": VOCAB, "width": width}
+
+
+def zusotar_dict(width, layers, heads, kv, dim, window, ldim, rot, lvdim, rank, gheads, gdim, gvdim, grank, experts, top,
+                 groups, keep, ff, shared, positions=4096) -> Dict[str, Any]:
+    moe = {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": shared},
+           "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+    mixers = [
+        ("attention", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                       "mask": {"size": window}}),
+        ("latent_attention", {"heads": heads, "dim": ldim, "rot_dim": rot, "vdim": lvdim, "kv_rank": rank,
+                              "scale": (ldim + rot) ** -0.5, "rot": {"base": 500000.0, "dims": rot}}),
+        ("gla", {"heads": gheads, "dim": gdim, "vdim": gvdim, "tau": 16.0, "decay_rank": grank}),
+    ]
+    ls = []
+    for i in range(layers):
+        kind, mixer = mixers[i % 3]
+        mlp = {"kind": "dense", "ff": 4 * width} if i == 0 and layers > 3 else json.loads(json.dumps(moe))
+        ls.append({"type": kind, "mixer": json.loads(json.dumps(mixer)), "mlp": mlp})
+    return {"architecture": "Zusotar", "layers": ls, "max_positions": positions, "norm": {"eps": 1e-5},
+            "residual_mult": 0.5, "vocab": VOCAB, "width": width}
 
 
 def moe_twin_config(lcfg, width, layers, heads, experts, top):
@@ -167,6 +199,29 @@ def run_pobelorn(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: 
     return 0
 
 
+def run_zusotar(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, dev) -> int:
+    from ..models.config import ModelConfig
+
+    for name in sizes:
+        z = ZUSOTAR_SIZES[name]
+        width, layers, heads, experts, top = z[0], z[1], z[2], z[14], z[15]
+        zcfg = ModelConfig.from_hf_dict(zusotar_dict(*z))
+        tcfg = moe_twin_config(zcfg, width, layers, heads, experts, top)
+        row = {"design": "zusotar", "size": name, "width": width, "layers": layers, "heads": heads, "kv_heads": z[3],
+               "head_dim": z[4], "window": z[5], "kv_rank": z[9], "rot_dim": z[7], "gla_heads": z[10], "gla_dim": z[11],
+               "gla_vdim": z[12], "experts": experts, "top": top, "groups": z[16], "groups_kept": z[17],
+               "expert_ff": z[18], "shared_ff": z[19], "twin_expert_ff": tcfg.moe_intermediate_size,
+               "prompts": n_prompts, "prompt_len": prompt_len, "new_tokens": new_tokens, "dtype": "bf16",
+               "data": "synthetic"}
+        for label, cfg in (("zusotar", zcfg), ("qwen3_moe_twin", tcfg)):
+            m = measure(cfg, n_prompts, prompt_len, new_tokens, dev)
+            row[label] = {"params_no_embedding": cfg.n_params(with_embedding=False), **{k: round(v, 1) for k, v in m.items()}}
+        row["prefill_ratio"] = round(row["zusotar"]["prefill_tok_s"] / row["qwen3_moe_twin"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["zusotar"]["decode_tok_s"] / row["qwen3_moe_twin"]["decode_tok_s"], 3)
+        print(json.dumps(row), flush=True)
+    return 0
+
+
 def run_lufivik(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, dev) -> int:
     from ..models.config import ModelConfig
 
@@ -195,6 +250,8 @@ def run(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, devi
         return run_lufivik(sizes, n_prompts, prompt_len, new_tokens, dev)
     if design == "pobelorn":
         return run_pobelorn(sizes, n_prompts, prompt_len, new_tokens, dev)
+    if design == "zusotar":
+        return run_zusotar(sizes, n_prompts, prompt_len, new_tokens, dev)
     for name in sizes:
         width, layers, heads, kv, dim, ff, window = SIZES[name]
         kcfg = ModelConfig.from_hf_dict(kuzanex_dict(width, layers, heads, kv, dim, ff, window))

@@ -770,24 +770,46 @@ class LogBiasWindowAttentionMixer(nn.Module):
         self.r2 = nn.Parameter(torch.zeros(heads, dtype=dtype, device=device))
         self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype, device=device))
         self.max_context = 1 << 30
+        self.standard = False  # the cache is in the engine's standard layout (`alloc_cache`)
 
     def cache_shape(self):
         return self.G, self.D, self.V
+
+    def alloc_cache(self, num_pages: int, dtype, device):
+        """Paged K / V of this layer: the engine's standard layout (and its flash / paged-decode kernels) for bf16
+        heads of 128 on the GPU, otherwise token-major pages of any key and value size."""
+        from ..ops.attention import alloc_kv_cache
+
+        self.standard = wattn.standard_layout_ok(self.D, self.V, dtype, device) and self.H // self.G <= 16
+        if self.standard:
+            return alloc_kv_cache(num_pages, self.G, self.D, dtype, device)
+        return wattn.alloc_window_cache(num_pages, self.G, self.D, self.V, dtype, device)
 
     def prepare(self, n_pos: int, tables: Dict[Any, torch.Tensor], device):
         self.max_context = int(n_pos) - 1
 
     def decode_splits(self, batch: int, max_context: int) -> int:
+        if self.standard:
+            from ..ops.attention import decode_num_splits
+
+            w = self.shape.window
+            return decode_num_splits(batch, self.G, max_context if w <= 0 else min(w + wattn.PAGE_SIZE, max_context))
         return wattn.decode_splits(batch, self.shape.window, max_context)
 
     def step(self, hc: torch.Tensor, st: StepTensors, cache) -> torch.Tensor:
         kc, vc = cache
         T = hc.shape[0]
         proj = F.linear(hc, self.proj)
-        q = wattn.qkv_vnorm_cache_write(proj, st.slots, kc, vc, self.H, self.eps, self.v_norm)
+        q = wattn.qkv_vnorm_cache_write(proj, st.slots, kc, vc, self.H, self.eps, self.v_norm,
+                                        v_transposed=self.standard, copy_q=not self.standard)
         nsplit = 1
         if st.max_q == 1 and st.nsplit > 1:
             nsplit = min(st.nsplit, self.decode_splits(T, self.max_context))
+        if self.standard:
+            o = wattn.window_attention_standard(q, kc, vc, st.block_tables, st.cu_q, st.cu_k, st.ctx_len, st.max_q,
+                                                self.shape, nsplit=nsplit, workspace=st.workspace,
+                                                log_bias=(self.r1, self.r2)).view(T, self.H * self.V)
+            return F.linear(wattn.sigmoid_gate_rows(o, proj[:, self.n_qkv:]), self.o)
         o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
                                    nsplit=nsplit, workspace=st.workspace, gate=proj[:, self.n_qkv:],
                                    log_bias=(self.r1, self.r2))

@@ -71,23 +71,27 @@ def qk_norm_cache_write(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_
 
 
 def qkv_vnorm_cache_write(proj: torch.Tensor, slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
-                          n_heads: int, eps: float, v_norm: bool = True) -> torch.Tensor:
+                          n_heads: int, eps: float, v_norm: bool = True, v_transposed: bool = False,
+                          copy_q: bool = True) -> torch.Tensor:
     """proj [T, >= (H + G) D + G Dv]: q heads | k heads | v heads (more columns may follow). Queries and keys stay as they
     are; with `v_norm` every value head is divided by its root mean square over Dv (no weight) and is cached so. Writes
-    k and v of tokens with slot >= 0 into the paged caches and returns the queries [T, H, D] (contiguous)."""
+    k and v of tokens with slot >= 0 into the paged caches (`v_transposed`: V pages [pages, G, Dv, 32]) and returns the
+    queries [T, H, D]: a contiguous copy, or (`copy_q` False) the view of proj that holds them."""
     T = proj.shape[0]
-    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[3]
+    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[2 if v_transposed else 3]
     H = n_heads
     assert proj.stride(1) == 1 and proj.shape[1] >= (H + G) * D + G * V
-    q = torch.empty(T, H, D, dtype=proj.dtype, device=proj.device)
+    q = torch.empty(T, H, D, dtype=proj.dtype, device=proj.device) if copy_q else proj[:, :H * D].view(T, H, D)
     if L.use_hip(proj):
         assert slots.dtype == torch.int64 and kcache.dtype == proj.dtype and vcache.dtype == proj.dtype
         L.check(L.lib().areal_qkv_vnorm_cache_write(
-            L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(slots), L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.c_int(T),
-            L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_float(eps), L.c_int(int(v_norm)),
-            L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "qkv_vnorm_cache_write")
+            L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(slots), L.ptr(q) if copy_q else None, L.ptr(kcache),
+            L.ptr(vcache), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_float(eps),
+            L.c_int(int(v_norm)), L.c_int(int(v_transposed)), L.c_int(L.dtype_flag(proj)), L.stream_ptr()),
+            "qkv_vnorm_cache_write")
         return q
-    q.copy_(proj[:, :H * D].reshape(T, H, D))
+    if copy_q:
+        q.copy_(proj[:, :H * D].reshape(T, H, D))
     ok = slots >= 0
     if ok.any():
         pg, off = (slots[ok] // PAGE_SIZE).long(), (slots[ok] % PAGE_SIZE).long()
@@ -95,8 +99,24 @@ def qkv_vnorm_cache_write(proj: torch.Tensor, slots: torch.Tensor, kcache: torch
         if v_norm:
             v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
         kcache[pg, :, off, :] = proj[ok, H * D:(H + G) * D].view(-1, G, D)
-        vcache[pg, :, off, :] = v.to(vcache.dtype)
+        if v_transposed:
+            vcache[pg, :, :, off] = v.to(vcache.dtype)
+        else:
+            vcache[pg, :, off, :] = v.to(vcache.dtype)
     return q
+
+
+def sigmoid_gate_rows(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x [T, n] (contiguous) <- x * sigmoid(gate) in place; gate [T, n], a view with unit stride along the columns."""
+    T, n = x.shape
+    assert x.is_contiguous() and gate.shape == x.shape and gate.stride(1) == 1 and gate.dtype == x.dtype
+    if L.use_hip(x):
+        L.check(L.lib().areal_sigmoid_gate_rows(L.ptr(x), L.ptr(gate), L.c_int64(gate.stride(0)), L.c_int64(T),
+                                                L.c_int(n), L.c_int(L.dtype_flag(x)), L.stream_ptr()),
+                "sigmoid_gate_rows")
+        return x
+    x.copy_((x.float() * torch.sigmoid(gate.float())).to(x.dtype))
+    return x
 
 
 def rotation_table(base: float, dims: int, n_pos: int, device, scaling: Optional[dict] = None) -> torch.Tensor:
@@ -191,15 +211,23 @@ def standard_layout_ok(dim: int, vdim: int, dtype, device) -> bool:
 def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: torch.Tensor, block_tables: torch.Tensor,
                               cu_q: torch.Tensor, cu_k: torch.Tensor, ctx_len: torch.Tensor, max_q: int,
                               shape: ScoreShape, nsplit: int = 1,
-                              workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                              workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                              log_bias: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
     """`window_attention` for layers in the standard cache layout (bf16, head size 128, V pages [pages, G, 128, 32]):
     plain scaled scores behind the window that keeps the first tokens. Prompt portions run the paged flash kernel,
     single-query rows the paged decode kernel (``csrc/hip/flash_attn_paged.hip``, ``csrc/hip/paged_attn.hip``), both
-    with the softmax weights at 16 bits of mantissa. cu_k int32 [B + 1]: cumulative context lengths."""
+    with the softmax weights at 16 bits of mantissa. cu_k int32 [B + 1]: cumulative context lengths. q may be a view
+    whose heads are contiguous. log_bias = (r1, r2), both [H]: r1_h ln(1 + r2_h (i - j)) is taken off the scaled score."""
     T, H, D = q.shape
     G = kcache.shape[1]
     B = cu_q.numel() - 1
-    assert L.use_hip(q) and q.dtype == torch.bfloat16 and D == 128 and vcache_t.shape[2] == 128 and q.is_contiguous()
+    assert L.use_hip(q) and q.dtype == torch.bfloat16 and D == 128 and vcache_t.shape[2] == 128
+    assert q.stride(2) == 1 and q.stride(1) == D
+    r1 = r2 = None
+    if log_bias is not None:
+        r1, r2 = log_bias
+        assert r1.dtype == q.dtype and r2.dtype == q.dtype and r1.numel() == H and r2.numel() == H
+        assert r1.is_contiguous() and r2.is_contiguous()
     assert shape.softcap <= 0 and shape.slope_exp == 0 and not shape.sink
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and ctx_len.dtype == torch.int32
     out = torch.empty(T, H, D, dtype=q.dtype, device=q.device)
@@ -216,14 +244,14 @@ def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: t
             L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.ptr(ctx_len), L.ptr(out), L.ptr(pa),
             L.ptr(pm), L.c_int(B), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(block_tables.shape[1]),
             L.c_int(int(nsplit)), L.c_float(shape.scale), L.c_int(q.stride(0)), L.c_int(int(shape.window)),
-            L.c_int(int(shape.keep_first)), L.stream_ptr()), "paged_decode_window")
+            L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.stream_ptr()), "paged_decode_window")
         return out
     assert cu_q.dtype == torch.int32 and cu_k.dtype == torch.int32
     L.check(L.lib().areal_flash_fwd_paged_window(
         L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(out),
         L.ptr(cu_q), L.ptr(cu_k), L.c_int(B), L.c_int(int(max_q)), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D),
         L.c_int64(q.stride(0)), L.c_int64(out.stride(0)), L.c_float(shape.scale), L.c_int(int(shape.window)),
-        L.c_int(int(shape.keep_first)), L.stream_ptr()), "flash_fwd_paged_window")
+        L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.stream_ptr()), "flash_fwd_paged_window")
     return out
 
 

@@ -105,10 +105,11 @@ def parse_args():
                         "beside a Qwen3-style transformer of equal size, one JSON line per size; comma-separated names "
                         "out of w1024, w2048, w4096, or 'all' (--prompts-per-gpu prompts of --prompt-len-max tokens, "
                         "--max-new-tokens new tokens each)")
-    p.add_argument("--serve-compare-design", default="kuzanex", choices=["kuzanex", "lufivik", "pobelorn"],
+    p.add_argument("--serve-compare-design", default="kuzanex", choices=["kuzanex", "lufivik", "pobelorn", "zusotar"],
                    help="the layer-list design --serve-compare measures: kuzanex beside a Qwen3-style twin, lufivik "
-                        "(latent attention, routed experts) or pobelorn (parallel blocks, window + lightning "
-                        "attention, routed + shared experts) beside a Qwen3-MoE-style twin")
+                        "(latent attention, routed experts), pobelorn (parallel blocks, window + lightning "
+                        "attention, routed + shared experts) or zusotar (depth-averaged layers of window, latent and "
+                        "gated linear attention, group-routed + shared experts) beside a Qwen3-MoE-style twin")
     a = p.parse_args()
     if a.seq_len:
         a.max_new_tokens = a.seq_len - a.prompt_len_max

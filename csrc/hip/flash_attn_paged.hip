@@ -31,7 +31,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
     const bf16_t* __restrict__ q, const void* __restrict__ kcache, const void* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, bf16_t* __restrict__ o, float* __restrict__ lse,
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, int64_t q_stride, int64_t o_stride, int Hq, int Hkv,
-    int nbatch, int total_q, float scale_log2, int causal, int window = 0, int keep = 0) {
+    int nbatch, int total_q, float scale_log2, int causal, int window = 0, int keep = 0,
+    const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr) {
   constexpr int D = 128;
   __shared__ __attribute__((aligned(16))) char smem[2 * 64 * 256];
   char* ks = smem;             // K tile  [64 keys][256 B], 16-byte chunks swizzled (flash_tiles.hpp)
@@ -73,6 +74,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
 #pragma unroll
     for (int j = 0; j < 16; ++j) oacc[i][j] = 0.f;
   float m = -INFINITY, l = 0.f;
+  // WIN with r1 / r2: r1_h ln(1 + r2_h (i - j)) is taken off the scaled score (in log2 units: r1_h log2(1 + r2_h (i - j)))
+  const bool biased = WIN && r1 != nullptr;
+  const float b1 = biased ? bf2f(r1[head]) : 0.f, b2 = biased ? bf2f(r2[head]) : 0.f;
 
   int k_hi = k_len;
   if (causal) {
@@ -164,6 +168,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         float sv = sacc[kb][j] * scale_log2;
+        if (biased) {
+          const int key = kbase + 32 * kb + (j & 3) + 8 * (j >> 2) + 4 * hf;
+          sv -= b1 * __log2f(1.f + b2 * (float)max(my_q + shift - key, 0));
+        }
         if (need_mask) {
           const int key = kbase + 32 * kb + (j & 3) + 8 * (j >> 2) + 4 * hf;
           if (key >= k_len || (causal && key > my_q + shift)) sv = -INFINITY;
@@ -260,12 +268,13 @@ extern "C" int areal_flash_fwd_paged(const void* q, const void* kcache, const vo
 }
 
 // The same over a sliding window that keeps the first `keep` tokens (window <= 0: every earlier key), bf16 caches,
-// softmax weights at 16 bits of mantissa; always causal.
+// softmax weights at 16 bits of mantissa; always causal. r1 / r2 (one number per query head each, or null): a learned
+// logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores.
 extern "C" int areal_flash_fwd_paged_window(const void* q, const void* kcache, const void* vcache,
                                             const int* block_tables, int max_pages, void* o, const int* cu_q,
                                             const int* cu_k, int B, int max_q, int total_q, int Hq, int Hkv, int D,
                                             int64_t q_stride, int64_t o_stride, float softmax_scale, int window, int keep,
-                                            hipStream_t st) {
+                                            const void* r1, const void* r2, hipStream_t st) {
   if (B == 0 || max_q == 0) return 0;
   if (D != 128) return -1;
   if (Hq % Hkv != 0) return -2;
@@ -276,6 +285,6 @@ extern "C" int areal_flash_fwd_paged_window(const void* q, const void* kcache, c
   dim3 grid((unsigned)(((max_q + 127) / 128) * (Hq / Hkv) * n_g_pad)), block(256);
   hipLaunchKernelGGL((flash_fwd_paged_kernel<false, true>), grid, block, 0, st, (const bf16_t*)q, kcache, vcache,
                      block_tables, max_pages, (bf16_t*)o, (float*)nullptr, cu_q, cu_k, q_stride, o_stride, Hq, Hkv, B,
-                     total_q, scale_log2, 1, window, keep);
+                     total_q, scale_log2, 1, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
   return (int)hipGetLastError();
 }

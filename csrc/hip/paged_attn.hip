@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
     const void* __restrict__ vcache, const int* __restrict__ block_tables,
     const int* __restrict__ context_lens, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int Hq, int Hkv, int max_pages, float scale_log2, int q_stride, int window = 0,
-    int keep = 0) {
+    int keep = 0, const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr) {
   constexpr int KS = D / 32;  // k-steps of the QK product
   constexpr int DB = D / 16;  // 16-wide d blocks of the PV product
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -70,6 +70,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
 #pragma unroll
   for (int i = 0; i < DB; ++i) o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;  // running max (log2 units) is shared by the 4 lanes of a q
+  // WIN with r1 / r2: r1_h log2(1 + r2_h (ctx - 1 - j)) is taken off the score of this lane's query head
+  const bool biased = WIN && r1 != nullptr && col < G;
+  const float b1 = biased ? bf2f(r1[h * G + col]) : 0.f, b2 = biased ? bf2f(r2[h * G + col]) : 0.f;
 
   const int* bt = block_tables + (size_t)b * max_pages;
   for (int pi = p_beg + wid; pi < p_end; pi += 4) {
@@ -101,7 +104,8 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
     float mx = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const float v = (r < 4 ? sa[r] : sb[r - 4]) * scale_log2;
+      float v = (r < 4 ? sa[r] : sb[r - 4]) * scale_log2;
+      if (WIN && r1 != nullptr) v -= b1 * __log2f(1.f + b2 * (float)max(ctx - 1 - (key0 + r), 0));
       s[r] = (key0 + r < ctx && (!windowed || ctx - 1 - (key0 + r) < window || key0 + r < keep)) ? v : -INFINITY;
       mx = fmaxf(mx, s[r]);
     }
@@ -268,11 +272,13 @@ extern "C" int areal_paged_decode(const void* q, const void* kcache, const void*
   return (int)hipGetLastError();
 }
 
-// Decode over a sliding window that keeps the first `keep` tokens; bf16 caches, head sizes 64 / 128.
+// Decode over a sliding window that keeps the first `keep` tokens; bf16 caches, head sizes 64 / 128. r1 / r2 (one number
+// per query head each, or null): a logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores.
 extern "C" int areal_paged_decode_window(const void* q, const void* kcache, const void* vcache, const int* block_tables,
                                          const int* context_lens, void* out, float* part_o, float* part_ml, int B,
                                          int Hq, int Hkv, int D, int max_pages, int nsplit, float softmax_scale,
-                                         int q_stride, int window, int keep, hipStream_t st) {
+                                         int q_stride, int window, int keep, const void* r1, const void* r2,
+                                         hipStream_t st) {
   if (B == 0) return 0;
   if (Hq % Hkv != 0 || Hq / Hkv > 16) return -1;
   if (D != 128 && D != 64) return -2;
@@ -282,11 +288,11 @@ extern "C" int areal_paged_decode_window(const void* q, const void* kcache, cons
   if (D == 128)
     hipLaunchKernelGGL((paged_decode_kernel<128, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
                        (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
-                       Hkv, max_pages, scale_log2, q_stride, window, keep);
+                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
   else
     hipLaunchKernelGGL((paged_decode_kernel<64, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
                        (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
-                       Hkv, max_pages, scale_log2, q_stride, window, keep);
+                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
   if (nsplit > 1)
     hipLaunchKernelGGL(paged_decode_reduce_kernel, dim3(B * Hq), dim3(D), 0, st, part_o, part_ml, (bf16_t*)out, nsplit, D);
   return (int)hipGetLastError();

@@ -224,7 +224,8 @@ __global__ void __launch_bounds__(256) rot_norm_cache_write_vec_kernel(
 template <typename T>
 __global__ void __launch_bounds__(256) qkv_vnorm_cache_write_kernel(
     const T* __restrict__ proj, int64_t row_stride, const int64_t* __restrict__ slots, T* __restrict__ q_out,
-    T* __restrict__ kcache, T* __restrict__ vcache, int H, int G, int D, int V, float eps, int v_norm) {
+    T* __restrict__ kcache, T* __restrict__ vcache, int H, int G, int D, int V, float eps, int v_norm,
+    int v_transposed) {
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * row_stride;
   const int64_t slot = slots[t];
@@ -233,7 +234,8 @@ __global__ void __launch_bounds__(256) qkv_vnorm_cache_write_kernel(
   const int off = slot >= 0 ? (int)(slot % PAGE) : 0;
   for (int u = blockIdx.y * 4 + wave; u < H + 2 * G; u += 4 * gridDim.y) {
     if (u < H) {
-      for (int d = lane; d < D; d += 64) q_out[((size_t)t * H + u) * D + d] = row[(size_t)u * D + d];
+      if (q_out)
+        for (int d = lane; d < D; d += 64) q_out[((size_t)t * H + u) * D + d] = row[(size_t)u * D + d];
     } else if (slot < 0) {
       continue;
     } else if (u < H + G) {
@@ -242,7 +244,9 @@ __global__ void __launch_bounds__(256) qkv_vnorm_cache_write_kernel(
     } else {
       const int c = u - H - G;
       const T* src = row + (size_t)(H + G) * D + (size_t)c * V;
-      T* dst = vcache + ((page * G + c) * PAGE + off) * V;
+      // V pages are [G][32][V], or [G][V][32] (a channel's 32 tokens side by side) for the kernels that want V^T
+      T* dst = v_transposed ? vcache + (page * G + c) * V * PAGE + off : vcache + ((page * G + c) * PAGE + off) * V;
+      const int dstep = v_transposed ? PAGE : 1;
       float r = 1.f;
       if (v_norm) {
         float ss = 0.f;
@@ -252,8 +256,20 @@ __global__ void __launch_bounds__(256) qkv_vnorm_cache_write_kernel(
         }
         r = 1.f / sqrtf(wave_sum(ss) / (float)V + eps);
       }
-      for (int d = lane; d < V; d += 64) stf<T>(dst, d, v_norm ? ldf<T>(src, d) * r : ldf<T>(src, d));
+      for (int d = lane; d < V; d += 64) stf<T>(dst, (size_t)d * dstep, v_norm ? ldf<T>(src, d) * r : ldf<T>(src, d));
     }
+  }
+}
+
+// x[t, i] *= sigmoid(gate[t, i]) over rows of n elements (x contiguous, gate rows gate_stride apart)
+template <typename T>
+__global__ void __launch_bounds__(256) sigmoid_gate_rows_kernel(T* __restrict__ x, const T* __restrict__ gate,
+                                                                int64_t gate_stride, int64_t rows, int n) {
+  const int64_t total = rows * n;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t t = i / n;
+    const float g = ldf<T>(gate, t * gate_stride + (i - t * n));
+    stf<T>(x, i, ldf<T>(x, i) / (1.f + expf(-g)));
   }
 }
 
@@ -763,15 +779,30 @@ extern "C" int areal_rot_norm_cache_write(const void* proj, int64_t row_stride, 
 // proj rows: q heads | k heads | v heads from the pointer on; nothing is rotated or normed but (v_norm) the values
 extern "C" int areal_qkv_vnorm_cache_write(const void* proj, int64_t row_stride, const int64_t* slots, void* q_out,
                                            void* kcache, void* vcache, int T, int H, int G, int D, int V, float eps,
-                                           int v_norm, int dt, hipStream_t st) {
+                                           int v_norm, int v_transposed, int dt, hipStream_t st) {
   if (T == 0) return 0;
   const dim3 grid(T, (H + 2 * G + 3) / 4);
   if (dt == 0)
     hipLaunchKernelGGL(qkv_vnorm_cache_write_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)proj, row_stride,
-                       slots, (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_norm);
+                       slots, (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache, H, G, D, V, eps, v_norm, v_transposed);
   else
     hipLaunchKernelGGL(qkv_vnorm_cache_write_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, row_stride,
-                       slots, (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps, v_norm);
+                       slots, (float*)q_out, (float*)kcache, (float*)vcache, H, G, D, V, eps, v_norm, v_transposed);
+  return (int)hipGetLastError();
+}
+
+// x [rows, n] contiguous <- x * sigmoid(gate), gate rows gate_stride apart
+extern "C" int areal_sigmoid_gate_rows(void* x, const void* gate, int64_t gate_stride, int64_t rows, int n, int dt,
+                                       hipStream_t st) {
+  if (rows == 0 || n == 0) return 0;
+  const int64_t total = rows * n;
+  const dim3 grid((unsigned)((total + 1023) / 1024 < 4096 ? (total + 1023) / 1024 : 4096));
+  if (dt == 0)
+    hipLaunchKernelGGL(sigmoid_gate_rows_kernel<bf16_t>, grid, dim3(256), 0, st, (bf16_t*)x, (const bf16_t*)gate,
+                       gate_stride, rows, n);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_rows_kernel<float>, grid, dim3(256), 0, st, (float*)x, (const float*)gate,
+                       gate_stride, rows, n);
   return (int)hipGetLastError();
 }
 
