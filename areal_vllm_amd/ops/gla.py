@@ -5,8 +5,9 @@ as fp32 state per request slot:
     S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,   o_t = S_t^T (q_t * q_scale)
     y_t = o_t / rms(o_t over V) * w * silu(g_t)                       per head, w [V] shared by the heads
 
-GPU: ``csrc/hip/gla.hip`` (token-by-token scan for decoding and short portions, chunks of 16 tokens for prompt
-portions). CPU: the same recurrence in PyTorch, token by token (fp32).
+GPU: ``csrc/hip/gla.hip`` (token-by-token scan for decoding and short portions; chunks of 16 tokens for prompt
+portions: one launch forms what does not depend on the state for all chunks at once, the next walks the chunks with
+matrix products only). CPU: the same recurrence in PyTorch, token by token (fp32).
 """
 from typing import Optional
 
@@ -14,6 +15,9 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib as L
+
+
+CHUNK = 16  # tokens per chunk of the chunked form
 
 
 def alloc_state(n_slots: int, n_heads: int, k_dim: int, v_dim: int, device) -> torch.Tensor:
@@ -41,10 +45,14 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Te
         if D > 256:
             raise RuntimeError("gated linear attention: key size above 256 is not built")
         obuf = torch.empty(T, NH, V, dtype=torch.float32, device=proj.device)
+        scratch = None
+        if max_q >= CHUNK and D <= 128:  # the chunked form's state-independent operands
+            scratch = torch.empty(T * (3 * NH * D + CHUNK * NH), dtype=torch.float32, device=proj.device)
         L.check(L.lib().areal_gla_scan(
             L.ptr(proj), L.c_int64(proj.stride(0)), L.c_int(q_off), L.c_int(k_off), L.c_int(v_off), L.ptr(z),
             L.c_int64(z.stride(0)), L.ptr(z_bias), L.c_float(tau), L.c_float(q_scale), L.ptr(cu_q), L.ptr(first_pos),
-            L.ptr(state_slots), L.ptr(state), L.ptr(obuf), L.c_int(B), L.c_int(NH), L.c_int(D), L.c_int(V),
+            L.ptr(state_slots), L.ptr(state), L.ptr(obuf), L.ptr(scratch), L.c_int(T), L.c_int(B), L.c_int(NH),
+            L.c_int(D), L.c_int(V),
             L.c_int(int(max_q)), L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "gla_scan")
         return obuf
     obuf = torch.zeros(T, NH, V, dtype=torch.float32, device=proj.device)

@@ -394,19 +394,37 @@ def test_gla_portions_rows_and_slots_used_again(device, dtype, H, D, V, tau, ran
     assert torch.equal(state[[1, 2]], before[[1, 2]])
 
 
-def test_gla_strong_decays_keep_every_exponent_finite():
+@pytest.mark.parametrize("device", DEVICES)
+def test_gla_strong_decays_keep_every_exponent_finite(device):
     """Logits far below zero with tau = 1 forget the state within a token: a chunked evaluation that divides by
     cumulative decays would overflow here."""
-    H, D, V, n = 1, 16, 8, 70
+    H, D, V, n = 2, 16, 8, 70
     g = torch.Generator().manual_seed(1)
     N = 2 * H * D + 2 * H * V
     rows = torch.randn(n, N, generator=g)
     z = torch.full((n, H * D), -60.0)
     z[:, ::3] = 5.0
-    state = gla_ops.alloc_state(1, H, D, V, "cpu")
-    o = gla_ops.gla_scan(rows, 0, H * D, 2 * H * D, z, None, 1.0, 0.25, i32([0, n], "cpu"), i32([0], "cpu"),
-                         i32([0], "cpu"), state, max_q=n)
+    z[40:, 1] = -200.0
+    eye = torch.eye(N, dtype=F64)
+    a, b, c = H * D, 2 * H * D, 2 * H * D + H * V
+    # the oracle forms its logits as a product: one input column of ones times the wanted logits
+    w = {"q": eye[:a], "k": eye[a:b], "v": eye[b:c], "g": eye[c:], "a1": torch.zeros(1, N, dtype=F64),
+         "a2": torch.zeros(H * D, 1, dtype=F64), "norm": torch.ones(V, dtype=F64), "o": torch.eye(H * V, dtype=F64)}
+    want = []
+    for t0, t1 in ((0, 40), (40, n)):  # the logits change once: two runs of the oracle, the state carried over
+        w["a2.b"] = z[t0].to(F64)
+        y, S = O.gla(rows[t0:t1].to(F64), w, "", {"heads": H, "dim": D, "vdim": V, "tau": 1.0}, 1e-5,
+                     state=None if t0 == 0 else S)
+        want.append(y)
+    want = torch.cat(want)
+    state = gla_ops.alloc_state(1, H, D, V, device)
+    rd = rows.to(device)
+    o = gla_ops.gla_scan(rd, 0, a, b, z.to(device), None, 1.0, D ** -0.5, i32([0, n], device), i32([0], device),
+                         i32([0], device), state, max_q=n)
     assert bool(torch.isfinite(o).all()) and bool(torch.isfinite(state).all())
+    got = gla_ops.gla_out(o, rd[:, c:], torch.ones(V, device=device), 1e-5)
+    assert rel_err(got.cpu(), want) < 2e-4
+    assert rel_err(state[0].reshape(1, -1).cpu(), S.reshape(1, -1)) < 1e-4
 
 
 @pytest.mark.parametrize("device", DEVICES)
