@@ -244,6 +244,61 @@ def test_window_edges_distance_penalty_gate_pages_portions_and_splits(device, dt
         assert rel_err(O.window_attention(seen(h, dtype), flat, "", m, 1e-6), want) > 0.1
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,window", [(4, 2, 70), (2, 1, 64), (4, 4, 200), (2, 2, 1000), (3, 1, 1), (16, 1, 33)])
+def test_standard_cache_layout_kernels_with_distance_penalty(H, G, window):
+    """bf16 heads of 128 live in the engine's standard cache (V pages transposed) and run its paged flash and paged
+    decode kernels with the distance penalty: window edges, page borders, portions and split key ranges."""
+    from areal_vllm_amd.ops.attention import alloc_kv_cache
+
+    D = V = 128
+    n, device, dtype = 200, "cuda", torch.bfloat16
+    pages = [3, 1, 4, 9, 2, 7, 5]
+    w_eff = min(window, n)
+
+    def run(h, w, m, portions, nsplit):
+        kc, vc = alloc_kv_cache(max(pages) + 2, G, D, dtype, device)
+        kc.fill_(50.0)
+        vc.fill_(-50.0)
+        shape = wattn.ScoreShape(scale=m["scale"], window=window)
+        bt = torch.tensor([pages], dtype=torch.int32, device=device)
+        r1, r2 = w["r1"].to(dtype).to(device), w["r2"].to(dtype).to(device)
+        hd = h.to(dtype).to(device)
+        outs, at = [], 0
+        for c in portions:
+            c = min(c, n - at)
+            if c <= 0:
+                break
+            rows = hd[at:at + c]
+            q = wattn.qkv_vnorm_cache_write(rows, _slots(pages, at, at + c, device), kc, vc, H, 1e-6, v_transposed=True,
+                                            copy_q=False)
+            assert q.data_ptr() == rows.data_ptr()
+            o = wattn.window_attention_standard(q, kc, vc, bt, i32([0, c], device), i32([0, at + c], device),
+                                                i32([at + c], device), c, shape, nsplit=nsplit if c == 1 else 1,
+                                                log_bias=(r1, r2)).view(c, H * V)
+            outs.append(wattn.sigmoid_gate_rows(o, rows[:, (H + G) * D + G * V:]).float().cpu())
+            at += c
+        return torch.cat(outs)
+
+    probes = []
+    for qi in (n - 1, 130, 97, 64, 63):
+        probes += [(qi, qi - w_eff + 1), (qi, qi - w_eff), (qi, 1), (qi, qi - 32), (qi, qi - 33)]
+    probes = [(a, b) for a, b in probes if 0 <= b <= a]
+    for k, (qi, kj) in enumerate(probes):
+        h, w, m = _window_case(H, G, D, V, window, 4.0 / math.sqrt(D) * 3, n, [(qi, kj)], 7 + k % 3)
+        hs = {key: (seen(val, dtype) if key in ("r1", "r2") else val) for key, val in w.items()}
+        want = O.window_attention(seen(h, dtype)[:qi + 1], hs, "", m, 1e-6)
+        for portions, nsplit in (([n], 1), ([qi, 1, n], 1), ([qi, 1, n], 3)):
+            got = run(h, w, m, portions, nsplit)
+            assert rel_err(got[qi:qi + 1], want[qi:qi + 1]) < tol(dtype), (qi, kj, portions, nsplit)
+    h, w, m = _window_case(H, G, D, V, window, 1.0 / math.sqrt(D), n, [], 1)
+    hs = {key: (seen(val, dtype) if key in ("r1", "r2") else val) for key, val in w.items()}
+    want = O.window_attention(seen(h, dtype), hs, "", m, 1e-6)
+    for portions in ([n], [1], [2], [3, 17, 1, 1, 64, 31, 2, 33, 48], [150, 1]):
+        got = run(h, w, m, portions + [portions[-1]] * n, 2)
+        assert rel_err(got, want) < tol(dtype), portions
+
+
 def _latent_case(H, D, P, V, R, n, seed, base=100.0, scale=None, far=None, sink=None):
     """One sequence whose projections are identity-like: the input's columns are the queries and the latent | rotary
     key. `far` = (query position, key position): that key's latent and rotary part are made to answer that query's
