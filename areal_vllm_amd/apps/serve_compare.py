@@ -108,8 +108,8 @@ def zusotar_dict(width, layers, heads, kv, dim, window, ldim, rot, lvdim, rank, 
         ("attention", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
                        "mask": {"size": window}}),
         ("latent_attention", {"heads": heads, "dim": ldim, "rot_dim": rot, "vdim": lvdim, "kv_rank": rank,
-                              "scale": (ldim + rot) ** -0.5, "rot": {"base": 500000.0, "dims": rot}}),
-        ("gla", {"heads": gheads, "dim": gdim, "vdim": gvdim, "tau": 16.0, "decay_rank": grank}),
+                              "scale": (ldim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}),
+        ("gla", {"heads": gheads, "dim": gdim, "vdim": gvdim, "tau": 8.0, "decay_rank": grank}),
     ]
     ls = []
     for i in range(layers):
