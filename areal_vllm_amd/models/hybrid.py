@@ -806,10 +806,13 @@ class LogBiasWindowAttentionMixer(nn.Module):
         if st.max_q == 1 and st.nsplit > 1:
             nsplit = min(st.nsplit, self.decode_splits(T, self.max_context))
         if self.standard:
+            gate = proj[:, self.n_qkv:]
+            fused = gate.stride(0) % 4 == 0 and gate.data_ptr() % 8 == 0  # the kernels read the gate as 8-byte vectors
             o = wattn.window_attention_standard(q, kc, vc, st.block_tables, st.cu_q, st.cu_k, st.ctx_len, st.max_q,
                                                 self.shape, nsplit=nsplit, workspace=st.workspace,
-                                                log_bias=(self.r1, self.r2)).view(T, self.H * self.V)
-            return F.linear(wattn.sigmoid_gate_rows(o, proj[:, self.n_qkv:]), self.o)
+                                                log_bias=(self.r1, self.r2),
+                                                gate=gate if fused else None).view(T, self.H * self.V)
+            return F.linear(o if fused else wattn.sigmoid_gate_rows(o, gate), self.o)
         o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, None,
                                    nsplit=nsplit, workspace=st.workspace, gate=proj[:, self.n_qkv:],
                                    log_bias=(self.r1, self.r2))

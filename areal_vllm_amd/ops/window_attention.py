@@ -212,12 +212,14 @@ def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: t
                               cu_q: torch.Tensor, cu_k: torch.Tensor, ctx_len: torch.Tensor, max_q: int,
                               shape: ScoreShape, nsplit: int = 1,
                               workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                              log_bias: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                              log_bias: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                              gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`window_attention` for layers in the standard cache layout (bf16, head size 128, V pages [pages, G, 128, 32]):
     plain scaled scores behind the window that keeps the first tokens. Prompt portions run the paged flash kernel,
     single-query rows the paged decode kernel (``csrc/hip/flash_attn_paged.hip``, ``csrc/hip/paged_attn.hip``), both
     with the softmax weights at 16 bits of mantissa. cu_k int32 [B + 1]: cumulative context lengths. q may be a view
-    whose heads are contiguous. log_bias = (r1, r2), both [H]: r1_h ln(1 + r2_h (i - j)) is taken off the scaled score."""
+    whose heads are contiguous. log_bias = (r1, r2), both [H]: r1_h ln(1 + r2_h (i - j)) is taken off the scaled score.
+    gate [T, H D] (a view with unit stride along the columns): the output times sigmoid(gate), element by element."""
     T, H, D = q.shape
     G = kcache.shape[1]
     B = cu_q.numel() - 1
@@ -230,6 +232,11 @@ def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: t
         assert r1.is_contiguous() and r2.is_contiguous()
     assert shape.softcap <= 0 and shape.slope_exp == 0 and not shape.sink
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and ctx_len.dtype == torch.int32
+    gstride = 0
+    if gate is not None:
+        assert gate.dtype == q.dtype and gate.shape == (T, H * D) and gate.stride(1) == 1
+        assert gate.stride(0) % 4 == 0 and gate.data_ptr() % 8 == 0
+        gstride = gate.stride(0)
     out = torch.empty(T, H, D, dtype=q.dtype, device=q.device)
     if max_q == 1:
         assert T == B
@@ -244,14 +251,16 @@ def window_attention_standard(q: torch.Tensor, kcache: torch.Tensor, vcache_t: t
             L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.ptr(ctx_len), L.ptr(out), L.ptr(pa),
             L.ptr(pm), L.c_int(B), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(block_tables.shape[1]),
             L.c_int(int(nsplit)), L.c_float(shape.scale), L.c_int(q.stride(0)), L.c_int(int(shape.window)),
-            L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.stream_ptr()), "paged_decode_window")
+            L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.ptr(gate), L.c_int64(gstride), L.stream_ptr()),
+            "paged_decode_window")
         return out
     assert cu_q.dtype == torch.int32 and cu_k.dtype == torch.int32
     L.check(L.lib().areal_flash_fwd_paged_window(
         L.ptr(q), L.ptr(kcache), L.ptr(vcache_t), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(out),
         L.ptr(cu_q), L.ptr(cu_k), L.c_int(B), L.c_int(int(max_q)), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D),
         L.c_int64(q.stride(0)), L.c_int64(out.stride(0)), L.c_float(shape.scale), L.c_int(int(shape.window)),
-        L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.stream_ptr()), "flash_fwd_paged_window")
+        L.c_int(int(shape.keep_first)), L.ptr(r1), L.ptr(r2), L.ptr(gate), L.c_int64(gstride), L.stream_ptr()),
+        "flash_fwd_paged_window")
     return out
 
 

@@ -32,7 +32,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
     const int* __restrict__ block_tables, int max_pages, bf16_t* __restrict__ o, float* __restrict__ lse,
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, int64_t q_stride, int64_t o_stride, int Hq, int Hkv,
     int nbatch, int total_q, float scale_log2, int causal, int window = 0, int keep = 0,
-    const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr) {
+    const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr,
+    const bf16_t* __restrict__ gate = nullptr, int64_t gate_stride = 0) {
   constexpr int D = 128;
   __shared__ __attribute__((aligned(16))) char smem[2 * 64 * 256];
   char* ks = smem;             // K tile  [64 keys][256 B], 16-byte chunks swizzled (flash_tiles.hpp)
@@ -233,8 +234,15 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_paged_kernel(
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         bf16x4 w;
+        if (WIN && gate) {  // one sigmoid gate per head and value channel of the token
+          const bf16x4 gv = *reinterpret_cast<const bf16x4*>(gate + (size_t)(q_beg + my_q) * gate_stride +
+                                                             (size_t)head * D + 32 * db + 8 * gq + 4 * hf);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w[j] = f2bf(oacc[db][4 * gq + j] * inv_l);
+          for (int j = 0; j < 4; ++j) w[j] = f2bf(oacc[db][4 * gq + j] * inv_l / (1.f + __expf(-bf2f(gv[j]))));
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) w[j] = f2bf(oacc[db][4 * gq + j] * inv_l);
+        }
         *reinterpret_cast<bf16x4*>(op + 32 * db + 8 * gq + 4 * hf) = w;
       }
     if (hf == 0 && lse)
@@ -269,22 +277,26 @@ extern "C" int areal_flash_fwd_paged(const void* q, const void* kcache, const vo
 
 // The same over a sliding window that keeps the first `keep` tokens (window <= 0: every earlier key), bf16 caches,
 // softmax weights at 16 bits of mantissa; always causal. r1 / r2 (one number per query head each, or null): a learned
-// logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores.
+// logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores. gate (rows of Hq 128 numbers, gate_stride
+// apart, or null): the output is multiplied by sigmoid(gate) element by element.
 extern "C" int areal_flash_fwd_paged_window(const void* q, const void* kcache, const void* vcache,
                                             const int* block_tables, int max_pages, void* o, const int* cu_q,
                                             const int* cu_k, int B, int max_q, int total_q, int Hq, int Hkv, int D,
                                             int64_t q_stride, int64_t o_stride, float softmax_scale, int window, int keep,
-                                            const void* r1, const void* r2, hipStream_t st) {
+                                            const void* r1, const void* r2, const void* gate, int64_t gate_stride,
+                                            hipStream_t st) {
   if (B == 0 || max_q == 0) return 0;
   if (D != 128) return -1;
   if (Hq % Hkv != 0) return -2;
   if ((q_stride | o_stride) % 8 != 0) return -3;
   if (((uintptr_t)q | (uintptr_t)kcache | (uintptr_t)vcache | (uintptr_t)o) % 16 != 0) return -4;
+  if (gate && (gate_stride % 4 != 0 || (uintptr_t)gate % 8 != 0)) return -5;
   const float scale_log2 = softmax_scale * 1.4426950408889634f;
   const int n_g_pad = (Hkv * B + 7) & ~7;
   dim3 grid((unsigned)(((max_q + 127) / 128) * (Hq / Hkv) * n_g_pad)), block(256);
   hipLaunchKernelGGL((flash_fwd_paged_kernel<false, true>), grid, block, 0, st, (const bf16_t*)q, kcache, vcache,
                      block_tables, max_pages, (bf16_t*)o, (float*)nullptr, cu_q, cu_k, q_stride, o_stride, Hq, Hkv, B,
-                     total_q, scale_log2, 1, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
+                     total_q, scale_log2, 1, window, keep, (const bf16_t*)r1, (const bf16_t*)r2, (const bf16_t*)gate,
+                     gate_stride);
   return (int)hipGetLastError();
 }

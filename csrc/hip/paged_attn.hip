@@ -38,7 +38,8 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
     const void* __restrict__ vcache, const int* __restrict__ block_tables,
     const int* __restrict__ context_lens, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int Hq, int Hkv, int max_pages, float scale_log2, int q_stride, int window = 0,
-    int keep = 0, const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr) {
+    int keep = 0, const bf16_t* __restrict__ r1 = nullptr, const bf16_t* __restrict__ r2 = nullptr,
+    const bf16_t* __restrict__ gate = nullptr, int64_t gate_stride = 0) {
   constexpr int KS = D / 32;  // k-steps of the QK product
   constexpr int DB = D / 16;  // 16-wide d blocks of the PV product
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -170,7 +171,10 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
     }
     const int head = h * G + qq;
     if (nsplit == 1) {
-      out[(size_t)b * Hq * D + (size_t)head * D + d] = f2bf(ll > 0.f ? acc / ll : 0.f);
+      float val = ll > 0.f ? acc / ll : 0.f;
+      // WIN with a gate: one sigmoid gate per head and value channel of the row
+      if (WIN && gate) val /= 1.f + __expf(-bf2f(gate[(size_t)b * gate_stride + (size_t)head * D + d]));
+      out[(size_t)b * Hq * D + (size_t)head * D + d] = f2bf(val);
     } else {
       part_o[(((size_t)b * Hq + head) * nsplit + split) * D + d] = acc;
       if (d == 0) {
@@ -186,7 +190,9 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void paged_decode_kernel(
 // chain of memory round trips (16 splits at a batch of 8 rows: 7.5 us for a few KB).
 __global__ void paged_decode_reduce_kernel(const float* __restrict__ part_o,
                                            const float* __restrict__ part_ml,
-                                           bf16_t* __restrict__ out, int nsplit, int D) {
+                                           bf16_t* __restrict__ out, int nsplit, int D,
+                                           const bf16_t* __restrict__ gate = nullptr, int64_t gate_stride = 0,
+                                           int Hq = 1) {
   constexpr int MAXS = 256;
   __shared__ float sm[MAXS], sl[MAXS];
   const int bh = blockIdx.x, d = threadIdx.x;
@@ -224,7 +230,9 @@ __global__ void paged_decode_reduce_kernel(const float* __restrict__ part_o,
     acc += po[(size_t)s * D] * f;
     ll += Lsum(s) * f;
   }
-  out[(size_t)bh * D + d] = f2bf(ll > 0.f ? acc / ll : 0.f);
+  float val = ll > 0.f ? acc / ll : 0.f;
+  if (gate) val /= 1.f + __expf(-bf2f(gate[(size_t)(bh / Hq) * gate_stride + (size_t)(bh % Hq) * D + d]));
+  out[(size_t)bh * D + d] = f2bf(val);
 }
 
 template <int D, bool FP8>
@@ -273,12 +281,13 @@ extern "C" int areal_paged_decode(const void* q, const void* kcache, const void*
 }
 
 // Decode over a sliding window that keeps the first `keep` tokens; bf16 caches, head sizes 64 / 128. r1 / r2 (one number
-// per query head each, or null): a logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores.
+// per query head each, or null): a logarithmic distance penalty r1_h ln(1 + r2_h (i - j)) on the scaled scores. gate
+// (rows of Hq D numbers, gate_stride apart, or null): the output is multiplied by sigmoid(gate) element by element.
 extern "C" int areal_paged_decode_window(const void* q, const void* kcache, const void* vcache, const int* block_tables,
                                          const int* context_lens, void* out, float* part_o, float* part_ml, int B,
                                          int Hq, int Hkv, int D, int max_pages, int nsplit, float softmax_scale,
                                          int q_stride, int window, int keep, const void* r1, const void* r2,
-                                         hipStream_t st) {
+                                         const void* gate, int64_t gate_stride, hipStream_t st) {
   if (B == 0) return 0;
   if (Hq % Hkv != 0 || Hq / Hkv > 16) return -1;
   if (D != 128 && D != 64) return -2;
@@ -288,13 +297,16 @@ extern "C" int areal_paged_decode_window(const void* q, const void* kcache, cons
   if (D == 128)
     hipLaunchKernelGGL((paged_decode_kernel<128, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
                        (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
-                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
+                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2,
+                       (const bf16_t*)gate, gate_stride);
   else
     hipLaunchKernelGGL((paged_decode_kernel<64, false, true>), dim3(B, Hkv, nsplit), dim3(256), lds, st,
                        (const bf16_t*)q, kcache, vcache, block_tables, context_lens, (bf16_t*)out, part_o, part_ml, Hq,
-                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2);
+                       Hkv, max_pages, scale_log2, q_stride, window, keep, (const bf16_t*)r1, (const bf16_t*)r2,
+                       (const bf16_t*)gate, gate_stride);
   if (nsplit > 1)
-    hipLaunchKernelGGL(paged_decode_reduce_kernel, dim3(B * Hq), dim3(D), 0, st, part_o, part_ml, (bf16_t*)out, nsplit, D);
+    hipLaunchKernelGGL(paged_decode_reduce_kernel, dim3(B * Hq), dim3(D), 0, st, part_o, part_ml, (bf16_t*)out, nsplit, D,
+                       (const bf16_t*)gate, gate_stride, Hq);
   return (int)hipGetLastError();
 }
 

@@ -273,10 +273,12 @@ def test_standard_cache_layout_kernels_with_distance_penalty(H, G, window):
             q = wattn.qkv_vnorm_cache_write(rows, _slots(pages, at, at + c, device), kc, vc, H, 1e-6, v_transposed=True,
                                             copy_q=False)
             assert q.data_ptr() == rows.data_ptr()
+            gate = rows[:, (H + G) * D + G * V:]
+            inside = (at // 7) % 2 == 0  # the gate inside the attention kernels, or as a launch of its own
             o = wattn.window_attention_standard(q, kc, vc, bt, i32([0, c], device), i32([0, at + c], device),
                                                 i32([at + c], device), c, shape, nsplit=nsplit if c == 1 else 1,
-                                                log_bias=(r1, r2)).view(c, H * V)
-            outs.append(wattn.sigmoid_gate_rows(o, rows[:, (H + G) * D + G * V:]).float().cpu())
+                                                log_bias=(r1, r2), gate=gate if inside else None).view(c, H * V)
+            outs.append((o if inside else wattn.sigmoid_gate_rows(o, gate)).float().cpu())
             at += c
         return torch.cat(outs)
 
